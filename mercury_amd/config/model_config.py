@@ -520,3 +520,225 @@ class LarozenConfig:
         if self.loops:
             out["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
         return out
+
+
+@dataclass(frozen=True)
+class DifferentialAttentionConfig:
+    """``layers[i].mixer`` of a Videdra layer of type ``attention``: grouped-query differential
+    attention (two score maps a head over the same values), a window that keeps the
+    sequence's first tokens, a gate per head; with ``kv_from`` the layer owns no key and value
+    projections and reads the cache of the layer named."""
+
+    heads: int
+    kv_heads: int
+    dim: int                 # per map
+    vdim: int
+    scale: float
+    diff: float
+    window: int = 0          # 0: every earlier token
+    keep_first: int = 0
+    rot_base: float = 10000.0
+    rot_dims: int = 0        # 0: queries and keys do not turn
+    kv_from: int | None = None
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "DifferentialAttentionConfig":
+        need = lambda key: _require_in(raw, key, where)
+        rot = raw.get("rot") or {}
+        mask = raw.get("mask") or {}
+        dim = int(need("dim"))
+        source = raw.get("kv_from")
+        cfg = cls(
+            heads=int(need("heads")), kv_heads=int(need("kv_heads")), dim=dim,
+            vdim=int(raw.get("vdim", dim)), scale=float(need("scale")), diff=float(need("diff")),
+            window=int(mask.get("size") or 0), keep_first=int(mask.get("keep_first") or 0),
+            rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", 0)),
+            kv_from=None if source is None else int(source))
+        for name in ("heads", "kv_heads", "dim", "vdim"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if cfg.heads % cfg.kv_heads:
+            raise ConfigError(f"{where}: {cfg.heads} heads are not a multiple of {cfg.kv_heads} kv_heads")
+        if cfg.rot_dims < 0 or cfg.rot_dims > cfg.dim or cfg.rot_dims % 2:
+            raise ConfigError(f"{where}.rot.dims {cfg.rot_dims} must be even and within dim {cfg.dim}")
+        if cfg.rot_dims and not cfg.rot_base > 0:
+            raise ConfigError(f"{where}.rot.base must be positive")
+        if cfg.window < 0 or cfg.keep_first < 0:
+            raise ConfigError(f"{where}.mask: size and keep_first are not negative")
+        return cfg
+
+    def same_cache_as(self, other: "DifferentialAttentionConfig") -> bool:
+        """Whether keys and values the other layer stores are what this one would store."""
+        mine = (self.heads, self.kv_heads, self.dim, self.vdim, self.rot_dims,
+                self.rot_base if self.rot_dims else 0.0)
+        theirs = (other.heads, other.kv_heads, other.dim, other.vdim, other.rot_dims,
+                  other.rot_base if other.rot_dims else 0.0)
+        return mine == theirs
+
+    def to_dict(self) -> dict:
+        out = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim,
+               "scale": self.scale, "diff": self.diff}
+        if self.window:
+            out["mask"] = {"size": self.window, "keep_first": self.keep_first}
+        if self.rot_dims:
+            out["rot"] = {"base": self.rot_base, "dims": self.rot_dims}
+        if self.kv_from is not None:
+            out["kv_from"] = self.kv_from
+        return out
+
+
+@dataclass(frozen=True)
+class RetentionConfig:
+    """``layers[i].mixer`` of a Videdra layer of type ``retention``."""
+
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+    rot_base: float = 10000.0
+    rot_dims: int = 0
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "RetentionConfig":
+        need = lambda key: _require_in(raw, key, where)
+        rot = raw.get("rot") or {}
+        dim = int(need("dim"))
+        cfg = cls(heads=int(need("heads")), dim=dim, vdim=int(raw.get("vdim", dim)),
+                  decay=tuple(float(g) for g in need("decay")),
+                  rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", 0)))
+        for name in ("heads", "dim", "vdim"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if len(cfg.decay) != cfg.heads:
+            raise ConfigError(f"{where}.decay lists {len(cfg.decay)} values for {cfg.heads} heads")
+        if any(not 0.0 <= g <= 1.0 for g in cfg.decay):
+            raise ConfigError(f"{where}.decay: every head's decay lies in [0, 1]")
+        if cfg.rot_dims < 0 or cfg.rot_dims > cfg.dim or cfg.rot_dims % 2:
+            raise ConfigError(f"{where}.rot.dims {cfg.rot_dims} must be even and within dim {cfg.dim}")
+        if cfg.rot_dims and not cfg.rot_base > 0:
+            raise ConfigError(f"{where}.rot.base must be positive")
+        return cfg
+
+    def to_dict(self) -> dict:
+        out = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "decay": list(self.decay)}
+        if self.rot_dims:
+            out["rot"] = {"base": self.rot_base, "dims": self.rot_dims}
+        return out
+
+
+@dataclass(frozen=True)
+class VidedraMlpConfig:
+    """``layers[i].mlp``: ``dense`` (one gated feed-forward of `ff`) or ``moe`` (`experts`
+    gated feed-forwards of `ff` of which a token uses `top`, and a shared one of `shared_ff`
+    when that is not 0)."""
+
+    kind: str
+    ff: int
+    experts: int = 0
+    top: int = 0
+    shared_ff: int = 0
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "VidedraMlpConfig":
+        kind = _require_in(raw, "kind", where)
+        if kind == "dense":
+            cfg = cls("dense", int(_require_in(raw, "ff", where)))
+        elif kind == "moe":
+            router = _require_in(raw, "router", where)
+            shared = raw.get("shared")
+            cfg = cls("moe", int(_require_in(_require_in(raw, "expert", where), "ff", where + ".expert")),
+                      experts=int(_require_in(router, "experts", where + ".router")),
+                      top=int(_require_in(router, "top", where + ".router")),
+                      shared_ff=int(_require_in(shared, "ff", where + ".shared")) if shared else 0)
+            if not 0 < cfg.top <= cfg.experts:
+                raise ConfigError(f"{where}.router: top {cfg.top} of {cfg.experts} experts")
+            if shared and cfg.shared_ff <= 0:
+                raise ConfigError(f"{where}.shared.ff must be positive")
+        else:
+            raise ConfigError(f"{where}.kind {kind!r} is not implemented; known: dense, moe")
+        if cfg.ff <= 0:
+            raise ConfigError(f"{where}: ff must be positive")
+        return cfg
+
+    def to_dict(self) -> dict:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff}
+        out = {"kind": "moe", "expert": {"ff": self.ff},
+               "router": {"experts": self.experts, "top": self.top}}
+        if self.shared_ff:
+            out["shared"] = {"ff": self.shared_ff}
+        return out
+
+
+@dataclass(frozen=True)
+class VidedraLayerConfig:
+    kind: str                                   # "attention" or "retention"
+    mixer: object                               # DifferentialAttentionConfig | RetentionConfig
+    mlp: VidedraMlpConfig | None
+
+
+@dataclass(frozen=True)
+class VidedraConfig:
+    """The Videdra decoder: layers with an RMS norm before and after each sublayer and a stored
+    vector per channel on what enters the float32 stream; a layer's mixer is a differential
+    attention (which may read an earlier layer's keys and values) or a retention with
+    per-request state; its feed-forward a tanh-gelu gated one, routed SiLU experts with a gated
+    shared expert, or none; an untied head behind a final norm."""
+
+    vocab: int
+    width: int
+    norm_eps: float
+    layers: tuple
+    architecture: str = "Videdra"
+    eos_token_ids: tuple = ()
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "VidedraConfig":
+        entries = _require(raw, "layers")
+        if not isinstance(entries, list) or not entries:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(entries):
+            where = f"layers[{i}]"
+            kind = _require_in(entry, "type", where)
+            mixer = _require_in(entry, "mixer", where)
+            if kind == "attention":
+                mixer_cfg = DifferentialAttentionConfig.from_dict(mixer, where + ".mixer")
+            elif kind == "retention":
+                mixer_cfg = RetentionConfig.from_dict(mixer, where + ".mixer")
+            else:
+                raise ConfigError(f"{where}.type {kind!r} is not implemented; known: attention, retention")
+            mlp = entry.get("mlp")
+            layers.append(VidedraLayerConfig(
+                kind, mixer_cfg, None if mlp is None else VidedraMlpConfig.from_dict(mlp, where + ".mlp")))
+        cfg = cls(vocab=int(_require(raw, "vocab")), width=int(_require(raw, "width")),
+                  norm_eps=float(_require_in(_require(raw, "norm"), "eps", "norm")),
+                  layers=tuple(layers),
+                  architecture=str(raw.get("architecture") or (raw.get("architectures") or ["Videdra"])[0]))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("vocab and width must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        for i, layer in enumerate(self.layers):
+            source = getattr(layer.mixer, "kv_from", None)
+            if source is None:
+                continue
+            where = f"layers[{i}].mixer.kv_from"
+            if not 0 <= source < i:
+                raise ConfigError(f"{where} {source} names no earlier layer")
+            other = self.layers[source]
+            if other.kind != "attention" or other.mixer.kv_from is not None:
+                raise ConfigError(f"{where}: layer {source} projects no keys and values of its own")
+            if not layer.mixer.same_cache_as(other.mixer):
+                raise ConfigError(f"{where}: layer {source} has other head counts, sizes or rotation")
+
+    def to_dict(self) -> dict:
+        return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
+                "norm": {"eps": self.norm_eps},
+                "layers": [{"type": layer.kind, "mixer": layer.mixer.to_dict(),
+                            "mlp": None if layer.mlp is None else layer.mlp.to_dict()}
+                           for layer in self.layers]}

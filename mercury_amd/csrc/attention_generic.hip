@@ -14,6 +14,9 @@
 // score_cap > 0 bounds it to cap * tanh(score / cap), and distance_slopes [n_q] subtracts
 // slope[head] * (query position - key position), a position encoding that lives in the score.
 // sinks [n_q] (float32, or null): exp(sink[head]) stands in the softmax's denominator once.
+// keep_first > 0 (with a window): the first keep_first keys of the sequence stay visible after
+// the window has passed them; they are walked first, in chunks of 64 from key 0, then the
+// window's keys from `first`.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -26,7 +29,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int table_stride, int page_shift, int n_q, int n_kv,
-    int d, int dv, float scale, int window, float score_cap,
+    int d, int dv, float scale, int window, int keep_first, float score_cap,
     const float* __restrict__ distance_slopes, const float* __restrict__ sinks) {
   __shared__ float qs[MAXD];
   __shared__ float probs[MK_WAVE];
@@ -47,10 +50,14 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
 #pragma unroll
   for (int c = 0; c < MAXD / MK_WAVE; ++c) acc[c] = 0.f;
 
-  for (int j0 = first; j0 <= pos; j0 += MK_WAVE) {
+  // two runs of keys: the kept first ones the window has passed, [0, kept), then [first, pos]
+  const int kept = min(keep_first, first);
+  for (int run = kept > 0 ? 0 : 1; run < 2; ++run) {
+  const int begin = run == 0 ? 0 : first, last = run == 0 ? kept - 1 : pos;
+  for (int j0 = begin; j0 <= last; j0 += MK_WAVE) {
     const int j = j0 + lane;
     float score = -INFINITY;
-    if (j <= pos) {
+    if (j <= last) {
       const int page = table[j >> page_shift];
       const T* krow =
           k_cache + (((size_t)page * n_kv + kvh) * page_size + (j & page_mask)) * d;
@@ -63,7 +70,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
       score -= slope * (float)(pos - j);
     }
     const float m_new = fmaxf(m, wave_max(score));
-    const float p = j <= pos ? expf(score - m_new) : 0.f;
+    const float p = j <= last ? expf(score - m_new) : 0.f;
     const float corr = expf(m - m_new);  // 0 on the first chunk, where m is -inf
     l = l * corr + wave_sum(p);
 #pragma unroll
@@ -71,7 +78,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     __syncthreads();
     probs[lane] = p;
     __syncthreads();
-    const int count = min(MK_WAVE, pos - j0 + 1);
+    const int count = min(MK_WAVE, last - j0 + 1);
     for (int jj = 0; jj < count; ++jj) {
       const int key = j0 + jj;
       const int page = table[key >> page_shift];
@@ -87,6 +94,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
       }
     }
     m = m_new;
+  }
   }
 
   // a sink: exp(sink[head]) once more in the denominator, with no key or value behind it
@@ -113,7 +121,8 @@ extern "C" int mk_attention_generic_kv(const void* q, int q_stride, void* out, i
                                        const int* positions, const int* token_seq,
                                        const int* block_table, int table_stride, int page_size,
                                        int n_q, int n_kv, int d, int dv, float scale, int window,
-                                       float score_cap, const float* distance_slopes,
+                                       int keep_first, float score_cap,
+                                       const float* distance_slopes,
                                        const float* sinks, int tokens, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv > 0 && d > 0 && dv > 0, "attention: bad sizes");
   MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
@@ -124,6 +133,7 @@ extern "C" int mk_attention_generic_kv(const void* q, int q_stride, void* out, i
   MK_REQUIRE(mk_is_pow2(page_size), "attention: page size %d is not a power of two", page_size);
   MK_REQUIRE(n_q <= 65535, "attention: too many heads (%d)", n_q);
   MK_REQUIRE(window >= 0, "attention: negative window");
+  MK_REQUIRE(keep_first >= 0, "attention: negative count of kept first keys");
   MK_REQUIRE(score_cap >= 0.f, "attention: negative score cap");
   if (tokens == 0) return 0;
   dim3 grid(tokens, n_q);
@@ -131,7 +141,7 @@ extern "C" int mk_attention_generic_kv(const void* q, int q_stride, void* out, i
   attention_generic_kernel<T, MAXD><<<grid, MK_WAVE, 0, stream>>>(                              \
       (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_cache, (const T*)v_cache,         \
       positions, token_seq, block_table, table_stride, mk_log2(page_size), n_q, n_kv, d, dv,    \
-      scale, window, score_cap, distance_slopes, sinks)
+      scale, window, keep_first, score_cap, distance_slopes, sinks)
   if (dtype == MK_F32) {
     if (widest <= AG_MAX_D) AG_LAUNCH(float, AG_MAX_D); else AG_LAUNCH(float, AG_MAX_WIDE);
   } else if (dtype == MK_BF16) {
@@ -155,5 +165,6 @@ extern "C" int mk_attention_generic(const void* q, int q_stride, void* out, int 
              AG_MAX_D);
   return mk_attention_generic_kv(q, q_stride, out, out_stride, k_cache, v_cache, dtype, positions,
                                  token_seq, block_table, table_stride, page_size, n_q, n_kv, d, d,
-                                 scale, window, score_cap, distance_slopes, nullptr, tokens, stream);
+                                 scale, window, 0, score_cap, distance_slopes, nullptr, tokens,
+                                 stream);
 }

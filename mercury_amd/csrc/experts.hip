@@ -14,7 +14,10 @@
 //
 // Gate activations (MK_ACT_*): SILU is round(silu(g)) * u as the SiLU-gated projection
 // computes it; SWISH_CLAMP is g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit),
-// u' = clamp(u, -limit, limit).
+// u' = clamp(u, -limit, limit); GELU_TANH is 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u.
+//
+//   mk_row_gate       act[t, :] *= sigmoid(x[t, :] . w): a feed-forward gated by one number a
+//                     token.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -22,6 +25,10 @@ template <typename T>
 __device__ __forceinline__ float gate_act(float g, float u, int kind, float limit, float alpha,
                                           float beta) {
   if (kind == MK_ACT_SILU) return Elem<T>::round(g / (1.f + expf(-g))) * u;
+  if (kind == MK_ACT_GELU_TANH) {
+    const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return 0.5f * g * (1.f + tanhf(inner)) * u;
+  }
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.f + expf(-alpha * g)) * (u + beta);
@@ -240,7 +247,8 @@ extern "C" int mk_expert_gated(const void* x, const void* w, int dtype, const in
                                int tokens, int top, int ff, int K, int kind, float limit,
                                float alpha, float beta, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && top > 0 && ff > 0 && K > 0, "expert_gated: bad sizes");
-  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP, "expert_gated: activation %d", kind);
+  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP || kind == MK_ACT_GELU_TANH,
+             "expert_gated: activation %d", kind);
   MK_REQUIRE((size_t)K * 4 <= 64 * 1024, "expert_gated: rows of %d are too wide", K);
   MK_REQUIRE((long long)tokens * top < (1ll << 31), "expert_gated: too many rows");
   if (tokens == 0) return 0;
@@ -299,7 +307,8 @@ __global__ void gate_act_kernel(const T* __restrict__ gate_up, T* __restrict__ o
 extern "C" int mk_gate_act(const void* gate_up, void* out, int dtype, int tokens, int inter,
                            int kind, float limit, float alpha, float beta, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && inter > 0, "gate_act: bad sizes T=%d I=%d", tokens, inter);
-  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP, "gate_act: activation %d", kind);
+  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP || kind == MK_ACT_GELU_TANH,
+             "gate_act: activation %d", kind);
   if (tokens == 0) return 0;
   const size_t total = (size_t)tokens * inter;
   size_t blocks = (total + 255) / 256;
@@ -360,5 +369,34 @@ extern "C" int mk_fill_zero(float* p, long long n, hipStream_t stream) {
   if (blocks > 65536) blocks = 65536;
   fill_zero_kernel<<<(int)blocks, 256, 0, stream>>>(p, (size_t)n);
   MK_LAUNCH_CHECK("fill_zero");
+  return 0;
+}
+
+// One workgroup per token: the dot product in float32, then the row scaled in place.
+template <typename T>
+__global__ __launch_bounds__(256) void row_gate_kernel(T* __restrict__ act, const T* __restrict__ x,
+                                                       const T* __restrict__ w, int inter,
+                                                       int hidden) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  float dot = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    dot = fmaf(Elem<T>::load(x + t * hidden + i), Elem<T>::load(w + i), dot);
+  const float gate = 1.f / (1.f + expf(-block_sum(dot, scratch)));
+  for (int i = threadIdx.x; i < inter; i += blockDim.x)
+    Elem<T>::store(act + t * inter + i, Elem<T>::load(act + t * inter + i) * gate);
+}
+
+extern "C" int mk_row_gate(void* act, const void* x, const void* w, int dtype, int tokens,
+                           int inter, int hidden, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && inter > 0 && hidden > 0, "row_gate: bad sizes");
+  if (tokens == 0) return 0;
+  if (dtype == MK_F32)
+    row_gate_kernel<float><<<tokens, 256, 0, stream>>>((float*)act, (const float*)x, (const float*)w, inter, hidden);
+  else if (dtype == MK_BF16)
+    row_gate_kernel<bf16_t><<<tokens, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)x, (const bf16_t*)w, inter, hidden);
+  else
+    MK_REQUIRE(false, "row_gate: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("row_gate");
   return 0;
 }

@@ -48,6 +48,10 @@ __device__ __forceinline__ float batched_act(float g, float u, const BatchedPara
     const float s = g / (1.f + __expf(-g));
     return bf16_to_f32(f32_to_bf16(s)) * u;
   }
+  if (p.act_kind == MK_ACT_GELU_TANH) {
+    const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return g / (1.f + __expf(-2.f * z)) * u;
+  }
   g = fminf(g, p.limit);
   u = fminf(fmaxf(u, -p.limit), p.limit);
   return g / (1.f + __expf(-p.alpha * g)) * (u + p.beta);
@@ -203,7 +207,8 @@ extern "C" int mk_expert_gated_mfma(const void* x, const void* w, void* act, con
   p.offsets = offsets;
   p.gather_div = top;
   p.act_kind = kind; p.limit = limit; p.alpha = alpha; p.beta = beta;
-  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP, "expert_gated: activation %d", kind);
+  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP || kind == MK_ACT_GELU_TANH,
+             "expert_gated: activation %d", kind);
   MK_REQUIRE(rows && offsets && top > 0, "expert_gated: no row lists");
   const int tiles = (max_rows + 15) / 16;
   if (batched_check(p, experts, tiles)) return 1;

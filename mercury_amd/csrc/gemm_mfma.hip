@@ -108,6 +108,11 @@ __device__ __forceinline__ float silu_for_bf16(float g) {
 // rounded once, by whoever stores it.
 __device__ __forceinline__ float gated_value(float g, float u, const QkvTarget& a) {
   if (a.act_kind == MK_ACT_SILU) return Elem<bf16_t>::round(silu_for_bf16(g)) * u;
+  if (a.act_kind == MK_ACT_GELU_TANH) {
+    // 0.5 g (1 + tanh(z)) = g / (1 + 2^(-2 z log2 e)), z = sqrt(2/pi) (g + 0.044715 g^3)
+    const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(z * -2.88539008177792681472f)) * u;
+  }
   g = fminf(g, a.act_limit);
   u = fminf(fmaxf(u, -a.act_limit), a.act_limit);
   return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * a.act_alpha * -1.44269504088896340736f)) *
@@ -707,7 +712,8 @@ extern "C" int mk_gated_skinny_act(const void* x, const void* w, void* act, int 
   MK_REQUIRE(M >= 1 && M <= 16, "gated projection: M=%d outside 1..16", M);
   MK_REQUIRE(inter > 0 && K > 0 && K % 8 == 0, "gated projection: K=%d must be a multiple of 8",
              K);
-  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP, "gated projection: activation %d", kind);
+  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP || kind == MK_ACT_GELU_TANH,
+             "gated projection: activation %d", kind);
   SkinnyArgs a = skinny_args(x, w, act, M, inter, K, (K + 127) / 128);
   a.act_kind = kind;
   a.act_limit = limit;
@@ -1414,7 +1420,8 @@ extern "C" int mk_gated_tiled(const void* x, const void* w, void* act, int M, in
 extern "C" int mk_gated_tiled_act(const void* x, const void* w, void* act, int M, int inter, int K,
                                   int config, int kind, float limit, float alpha, float beta,
                                   hipStream_t stream) {
-  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP, "gated projection: activation %d", kind);
+  MK_REQUIRE(kind == MK_ACT_SILU || kind == MK_ACT_SWISH_CLAMP || kind == MK_ACT_GELU_TANH,
+             "gated projection: activation %d", kind);
   QkvTarget target = QkvTarget();
   target.act_kind = kind;
   target.act_limit = limit;

@@ -178,8 +178,23 @@ bool CacheManager::grow(const std::string& key, int start, int new_len) {
     if (spec.window != 0 && (int)table.size() < want) {
       // Pages wholly before the window of the first new query are never read.
       const int skip_to = std::min(first_needed(spec, start) / page_size_, want);
+      const int kept = kept_pages(spec);
       skipped.push_back({g, (int)table.size(), seq.first_live[g]});
-      while ((int)table.size() < skip_to) table.push_back(-1);
+      while ((int)table.size() < skip_to && ok) {
+        if ((int)table.size() >= kept) {
+          table.push_back(-1);
+          continue;
+        }
+        // a page of kept first tokens is held like any page of the window
+        const int page = groups_[g].pool->take();
+        if (page < 0) {
+          ok = false;
+          break;
+        }
+        table.push_back(page);
+        added.emplace_back(g, page);
+      }
+      if (!ok) break;
       seq.first_live[g] = std::max(seq.first_live[g], std::min(skip_to, (int)table.size()));
     }
     while ((int)table.size() < want) {
@@ -212,7 +227,7 @@ int CacheManager::trim(const std::string& key, int num_computed) {
     if (spec.window == 0) continue;
     std::vector<int>& table = seq.tables[g];
     const int keep_from = std::min(first_needed(spec, num_computed) / page_size_, (int)table.size());
-    for (int index = seq.first_live[g]; index < keep_from; ++index) {
+    for (int index = std::max(seq.first_live[g], kept_pages(spec)); index < keep_from; ++index) {
       if (table[index] >= 0) {
         groups_[g].pool->give_back(&table[index], 1);
         table[index] = -1;

@@ -10,6 +10,8 @@
 //     grows across a page edge.
 //   * A group with a window takes pages step by step, for the tokens of the step, and gives
 //     back every page whose last position the window has passed; the table keeps -1 there.
+//     A window that keeps the sequence's first tokens visible (keep_first) never gives back,
+//     or skips, the pages that hold them.
 //   * Everything goes back to its pool when the sequence ends, is aborted or is preempted.
 // Prefix sharing needs every group to keep all keys and no mixer to carry state of its own;
 // otherwise a cached page does not describe all that a later sequence needs.
@@ -28,9 +30,10 @@ struct GroupSpec {
   int kv_heads = 0, k_dim = 0, v_dim = 0;
   int dtype = -1;      // element type of keys and values; -1: the model's compute dtype
   int window = 0;      // 0: all earlier keys
+  int keep_first = 0;  // with a window: the first tokens stay visible after it has passed them
   bool operator==(const GroupSpec& o) const {
     return kv_heads == o.kv_heads && k_dim == o.k_dim && v_dim == o.v_dim && dtype == o.dtype &&
-           window == o.window;
+           window == o.window && (window == 0 || keep_first == o.keep_first);
   }
 };
 
@@ -117,6 +120,10 @@ class CacheManager {
  private:
   static int first_needed(const GroupSpec& spec, int next_position) {
     return spec.window == 0 ? 0 : std::max(0, next_position - spec.window + 1);
+  }
+  // Pages from the table's start that a window never passes.
+  int kept_pages(const GroupSpec& spec) const {
+    return spec.window == 0 ? 0 : (spec.keep_first + page_size_ - 1) / page_size_;
   }
   Sequence& mutable_sequence(const std::string& key);
 

@@ -94,18 +94,22 @@ py::dict pool_stats(const PagePool& pool) {
 GroupSpec spec_from_py(const py::handle& obj) {
   py::tuple t = py::hasattr(obj, "as_tuple") ? py::tuple(obj.attr("as_tuple")())
                                               : py::reinterpret_borrow<py::tuple>(obj);
-  if (t.size() != 5) throw py::value_error("a cache need is (kv_heads, k_dim, v_dim, dtype, window)");
+  if (t.size() != 5 && t.size() != 6) {
+    throw py::value_error("a cache need is (kv_heads, k_dim, v_dim, dtype, window[, keep_first])");
+  }
   GroupSpec s;
   s.kv_heads = py::cast<int>(t[0]);
   s.k_dim = py::cast<int>(t[1]);
   s.v_dim = py::cast<int>(t[2]);
   s.dtype = py::cast<int>(t[3]);
   s.window = py::cast<int>(t[4]);
+  s.keep_first = t.size() > 5 ? py::cast<int>(t[5]) : 0;
+  if (s.keep_first < 0) throw py::value_error("a cache need keeps no negative number of first tokens");
   return s;
 }
 
 py::tuple spec_to_py(const GroupSpec& s) {
-  return py::make_tuple(s.kv_heads, s.k_dim, s.v_dim, s.dtype, s.window);
+  return py::make_tuple(s.kv_heads, s.k_dim, s.v_dim, s.dtype, s.window, s.keep_first);
 }
 
 SchedulerOptions scheduler_options(const std::string& policy, int max_running, int prefill_budget,

@@ -10,11 +10,12 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 31
+#define MK_ABI_VERSION 32
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
-// g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit).
-enum { MK_ACT_SILU = 0, MK_ACT_SWISH_CLAMP = 1 };
+// g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit);
+// GELU_TANH is 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u.
+enum { MK_ACT_SILU = 0, MK_ACT_SWISH_CLAMP = 1, MK_ACT_GELU_TANH = 2 };
 // Activations of one operand: the square of relu.
 enum { MK_UNARY_RELU2 = 0 };
 
@@ -120,12 +121,13 @@ int mk_fill_normal(void* out, int dtype, long long n, unsigned long long key, fl
 // mk_attention_generic with keys of width d and values of width dv (the value cache is
 // [pages, n_kv, dv, page_size]); the output rows hold n_q heads of dv.  sinks (float32 [n_q],
 // or null): exp(sink[head]) is added once to the softmax's denominator, unscaled, with no key
-// or value behind it.
+// or value behind it.  keep_first (with a window): the sequence's first keep_first keys stay
+// visible to queries whose window has passed them.
 int mk_attention_generic_kv(const void* q, int q_stride, void* out, int out_stride,
                             const void* k_cache, const void* v_cache, int dtype,
                             const int* positions, const int* token_seq, const int* block_table,
                             int table_stride, int page_size, int n_q, int n_kv, int d, int dv,
-                            float scale, int window, float score_cap,
+                            float scale, int window, int keep_first, float score_cap,
                             const float* distance_slopes, const float* sinks, int tokens,
                             hipStream_t stream);
 
@@ -177,6 +179,11 @@ int mk_expert_gated(const void* x, const void* w, int dtype, const int* ids, voi
 int mk_expert_down(const void* act, const void* w, int dtype, const int* ids, const float* weights,
                    float* y, int tokens, int top, int ff, int N, hipStream_t stream);
 
+// act[t, :] *= sigmoid(x[t, :] . w) in place: a feed-forward's activations (`dtype`, [T, inter])
+// scaled by a gate of one number per token, the dot product and the sigmoid in float32.
+int mk_row_gate(void* act, const void* x, const void* w, int dtype, int tokens, int inter,
+                int hidden, hipStream_t stream);
+
 // out[t, i] = gate_act(gate_up[t, i], gate_up[t, I + i]) for an activation MK_ACT_*.
 int mk_gate_act(const void* gate_up, void* out, int dtype, int tokens, int inter, int kind,
                 float limit, float alpha, float beta, hipStream_t stream);
@@ -204,13 +211,17 @@ int mk_fill_zero(float* p, long long n, hipStream_t stream);
 // (temp_every 0: none); the first `rot` dims of every head turned as in mk_rope_kv_write.
 // q goes to q_out [T, n_q d] of `dtype`, k and v into the paged cache (values [pages, n_kv, dv,
 // page_size]) when write_kv.
+// maps > 1: a head of d dims is `maps` score maps of d / maps dims side by side, each turned in
+// its own first `rot` dims; q_out is then [T, n_q maps, d], query (head, map) holding its
+// map's dims in their place and zeros elsewhere, so that its product with a whole key row is
+// the map's score.
 int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int dtype, const void* q_norm,
                   const void* k_norm, int norm_dtype, float eps, float temp_coef, int temp_every,
                   const float* cos_table, const float* sin_table, int table_positions, int rot,
                   int interleaved, const int* positions, const int* token_seq,
                   const int* block_table, int table_stride, void* k_cache, void* v_cache,
                   int page_size, int n_q, int n_kv, int d, int dv, int values_are_keys,
-                  int write_kv, int tokens, hipStream_t stream);
+                  int write_kv, int maps, int tokens, hipStream_t stream);
 
 // out[i] = act(x[i]) for an activation MK_UNARY_*; x of in_dtype (float32, or the output's),
 // the result rounded once to `dtype`.
@@ -223,6 +234,21 @@ int mk_unary_act(const void* x, int in_dtype, void* out, int dtype, long long n,
 int mk_normed_sum(float* h, const float* ya, const float* pa, int na, const void* wa,
                   const float* yb, const float* pb, int nb, const void* wb, int weight_dtype,
                   float eps, float mult, long long stride, int tokens, int hidden,
+                  hipStream_t stream);
+
+// h[t, :] += scale .* (rmsnorm(y[t, :] + its `count` partial sums p[k * stride + .]) * weight):
+// a sublayer's output normed before it enters the stream, times a stored vector per channel
+// (`scale`, float32 or null).
+int mk_norm_scale_add(float* h, const float* y, const float* partials, int count,
+                      long long stride, const void* weight, int weight_dtype, const float* scale,
+                      float eps, int tokens, int hidden, hipStream_t stream);
+
+// Differential attention's tail.  a [T, heads, 2, dv] (`dtype`) holds two maps' outputs per
+// head; o = a1 - lambda * a2 is divided by its root mean square over dv (eps inside the root),
+// multiplied by out_scale and, when gate is not null, by sigmoid(gate[t * gate_stride + head])
+// (float32); out [T, heads dv] of `dtype`.
+int mk_diff_heads(const void* a, void* out, int dtype, const float* gate, int gate_stride,
+                  float lambda, float eps, float out_scale, int tokens, int heads, int dv,
                   hipStream_t stream);
 
 // out[t, :] = [a[t, :] | b[t, :]] in `dtype`; mk_copy_f32: dst[i] = src[i] by a kernel.
@@ -257,6 +283,22 @@ int mk_ssm_scan(const float* xbc, int xbc_stride, const float* proj, int proj_st
 int mk_ssm_chunk_tokens();
 long long mk_ssm_scan_workspace(int total_chunks, int heads, int P, int N);
 long long mk_ssm_state_floats(int heads, int P, int N);
+// Retention: per head S_t = decay S_(t-1) + k_t v_t^T (S is dim x vdim, float32), o_t = S_t^T q_t.
+// q, k, v are columns q_col, k_col, v_col of the float32 rows of proj ([heads dim], [heads dim],
+// [heads vdim]); the first `rot` dims of every q and k head turn by the tabulated angles of the
+// token's position (dim j with j + rot / 2), and k is multiplied by k_scale after the turn.
+// The state of a sequence is its slot's row of `state` ([heads, dim, vdim], rows slot_stride
+// floats apart), read at the step's start and left for the next; out [T, heads vdim] float32.
+int mk_retention_scan(const float* proj, int proj_stride, int q_col, int k_col, int v_col,
+                      const float* decay, float k_scale, const float* cos_table,
+                      const float* sin_table, int table_positions, int rot, const int* positions,
+                      const int* cu_q, const int* slots, float* state, long long slot_stride,
+                      int heads, int dim, int vdim, float* out, int tokens, int num_seqs,
+                      hipStream_t stream);
+// out[t, head, :] = y[t, head, :] / rms(y[t, head, :]) * silu(gate[t * gate_stride + head dv + .]):
+// a norm per head without a weight, then a gate (float32 columns of a projection).
+int mk_head_norm_gate(const float* y, void* out, int dtype, const float* gate, int gate_stride,
+                      float eps, int tokens, int heads, int dv, hipStream_t stream);
 // out[t, part] = y[t, part] / rms(y[t, part]) * weight[part], the row in `parts` equal parts.
 int mk_group_rmsnorm(const float* y, void* out, int dtype, const void* weight, int weight_dtype,
                      float eps, int tokens, int width, int parts, hipStream_t stream);

@@ -7,6 +7,9 @@
 //                      cache (the values may be the keys as projected);
 //   mk_unary_act       an activation of one operand (the square of relu);
 //   mk_normed_sum      h += mult * (rmsnorm(a) * wa + rmsnorm(b) * wb): mixers side by side;
+//   mk_norm_scale_add  h += scale .* (rmsnorm(y) * w): a sublayer's output normed before it
+//                      enters the stream, times a stored vector per channel;
+//   mk_diff_heads      two attention maps per head combined, normed per head and gated;
 //   mk_concat_cast     [a | b] row by row, in the compute dtype (the operand of a projection
 //                      of two streams);
 //   mk_copy_f32        a copy by a kernel (a captured graph records no memcpy node here).
@@ -32,7 +35,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     int rot, int interleaved, const int* __restrict__ positions,
     const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int page_shift, int n_q, int n_kv, int d,
-    int dv, int values_are_keys, int write_kv) {
+    int dv, int values_are_keys, int write_kv, int maps) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const int pos = positions[t];
@@ -67,8 +70,15 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const float v = k_src[i] * k_mult;
     return k_norm ? v * weight_at<TW>(k_norm, i) : v;
   };
-  // entry j of a head after the turn: the partner is j ^ 1 (interleaved) or j -+ half
+  // entry j of a head after the turn: the partner is j ^ 1 (interleaved) or j -+ half; a head
+  // of several score maps turns each map's first dims by itself
+  const int map_dims = d / maps;
   auto turned = [&](auto at, int base, int j) {
+    if (maps > 1) {
+      const int map = j / map_dims;
+      base += map * map_dims;
+      j -= map * map_dims;
+    }
     if (j >= rot) return at(base + j);
     if (interleaved) {
       const int pair = j >> 1;
@@ -87,19 +97,22 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   const int off = pos & (page_size - 1);
   // (the host never schedules a write into a page that was given back: page < 0 writes nothing)
   const int vw = n_kv * dv;
-  const int total = qw + (write_kv && page >= 0 ? kw + vw : 0);
+  const int qo = qw * maps;      // queries out: one per (head, map), a key row wide
+  const int total = qo + (write_kv && page >= 0 ? kw + vw : 0);
   const float* v_src = values_are_keys ? k_src : k_src + kw;
   for (int idx = blockIdx.y * blockDim.x + threadIdx.x; idx < total; idx += gridDim.y * blockDim.x) {
-    if (idx < qw) {
-      const int head = idx / d, j = idx - head * d;
-      Elem<T>::store(q_out + (size_t)t * qw + idx, turned(q_at, head * d, j));
-    } else if (idx < qw + kw) {
-      const int i = idx - qw;
+    if (idx < qo) {
+      const int query = idx / d, j = idx - query * d;
+      const int head = query / maps, map = query - head * maps;
+      const bool mine = maps == 1 || j / map_dims == map;
+      Elem<T>::store(q_out + (size_t)t * qo + idx, mine ? turned(q_at, head * d, j) : 0.f);
+    } else if (idx < qo + kw) {
+      const int i = idx - qo;
       const int head = i / d, j = i - head * d;
       const size_t dst = (((size_t)page * n_kv + head) * page_size + off) * d + j;
       Elem<T>::store(k_cache + dst, turned(k_at, head * d, j));
     } else {
-      const int i = idx - qw - kw;
+      const int i = idx - qo - kw;
       const int head = i / dv, j = i - head * dv;
       Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * dv + j) * page_size + off, v_src[i]);
     }
@@ -154,6 +167,53 @@ __global__ __launch_bounds__(256) void normed_sum_kernel(
   }
 }
 
+// One workgroup per token (or several that share its outputs, each making the sum of squares
+// for itself in the same order).
+template <typename TW>
+__global__ __launch_bounds__(256) void norm_scale_add_kernel(
+    float* __restrict__ h, const float* __restrict__ y, const float* __restrict__ partials,
+    int count, size_t stride, const void* __restrict__ weight, const float* __restrict__ scale,
+    float eps, int hidden) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * hidden;
+  auto value = [&](int i) {
+    float v = y ? y[base + i] : 0.f;
+    for (int k = 0; k < count; ++k) v += partials[(size_t)k * stride + base + i];
+    return v;
+  };
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = value(i);
+    sq += v * v;
+  }
+  const float r = rsqrtf(block_sum(sq, scratch) / (float)hidden + eps);
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < hidden; i += gridDim.y * blockDim.x) {
+    const float normed = value(i) * r * weight_at<TW>(weight, i);
+    h[base + i] += scale ? scale[i] * normed : normed;
+  }
+}
+
+// One wavefront per (token, head).
+template <typename T>
+__global__ __launch_bounds__(64) void diff_heads_kernel(
+    const T* __restrict__ a, T* __restrict__ out, const float* __restrict__ gate, int gate_stride,
+    float lambda, float eps, float out_scale, int heads, int dv) {
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const T* a1 = a + ((size_t)t * heads + head) * 2 * dv;
+  const T* a2 = a1 + dv;
+  float sq = 0.f;
+  for (int i = lane; i < dv; i += MK_WAVE) {
+    const float o = Elem<T>::load(a1 + i) - lambda * Elem<T>::load(a2 + i);
+    sq += o * o;
+  }
+  float mult = rsqrtf(wave_sum(sq) / (float)dv + eps) * out_scale;
+  if (gate) mult *= 1.f / (1.f + expf(-gate[(size_t)t * gate_stride + head]));
+  for (int i = lane; i < dv; i += MK_WAVE) {
+    const float o = Elem<T>::load(a1 + i) - lambda * Elem<T>::load(a2 + i);
+    Elem<T>::store(out + ((size_t)t * heads + head) * dv + i, o * mult);
+  }
+}
+
 template <typename T>
 __global__ void concat_cast_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                    T* __restrict__ out, int hidden) {
@@ -179,10 +239,13 @@ extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int 
                              int interleaved, const int* positions, const int* token_seq,
                              const int* block_table, int table_stride, void* k_cache,
                              void* v_cache, int page_size, int n_q, int n_kv, int d, int dv,
-                             int values_are_keys, int write_kv, int tokens, hipStream_t stream) {
+                             int values_are_keys, int write_kv, int maps, int tokens,
+                             hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv >= 0 && d > 0 && dv > 0, "qk_prepare: bad sizes");
-  MK_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0,
-             "qk_prepare: rotary width %d not in [0, %d] / even", rot, d);
+  MK_REQUIRE(maps >= 1 && d % maps == 0, "qk_prepare: %d maps do not divide a head of %d", maps, d);
+  MK_REQUIRE(rot >= 0 && rot <= d / maps && rot % 2 == 0,
+             "qk_prepare: rotary width %d not in [0, %d] / even", rot, d / maps);
+  MK_REQUIRE(maps == 1 || !interleaved, "qk_prepare: several maps turn in the half-split layout");
   MK_REQUIRE(rot == 0 || (table_positions > 0 && cos_table && sin_table),
              "qk_prepare: empty angle table");
   MK_REQUIRE(mk_is_pow2(page_size), "qk_prepare: page size %d is not a power of two", page_size);
@@ -197,14 +260,14 @@ extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int 
   MK_REQUIRE(norm_dtype == MK_F32 || norm_dtype == MK_BF16, "qk_prepare: norm dtype %d", norm_dtype);
   if (tokens == 0) return 0;
   // few tokens: a token's outputs over several workgroups, so that the chip is not idle
-  const int by_size = (need + 255) / 256;
+  const int by_size = (need + n_q * d * (maps - 1) + 255) / 256;
   const int chunks = std::max(1, std::min(by_size, 1024 / tokens));
   const dim3 grid(tokens, chunks);
 #define QK_LAUNCH(T, TW)                                                                         \
   qk_prepare_kernel<T, TW><<<grid, 256, 0, stream>>>(                                          \
       qkv, row_stride, (T*)q_out, q_norm, k_norm, eps, temp_coef, temp_every, cos_table,         \
       sin_table, rot, interleaved, positions, token_seq, block_table, table_stride, (T*)k_cache, \
-      (T*)v_cache, mk_log2(page_size), n_q, n_kv, d, dv, values_are_keys, write_kv)
+      (T*)v_cache, mk_log2(page_size), n_q, n_kv, d, dv, values_are_keys, write_kv, maps)
   if (dtype == MK_F32) {
     if (norm_dtype == MK_F32) QK_LAUNCH(float, float); else QK_LAUNCH(float, bf16_t);
   } else if (dtype == MK_BF16) {
@@ -256,6 +319,47 @@ extern "C" int mk_normed_sum(float* h, const float* ya, const float* pa, int na,
     normed_sum_kernel<bf16_t><<<grid, 256, 0, stream>>>(h, ya, pa, na, wa, yb, pb, nb, wb, eps,
                                                            mult, (size_t)stride, hidden);
   MK_LAUNCH_CHECK("normed_sum");
+  return 0;
+}
+
+extern "C" int mk_norm_scale_add(float* h, const float* y, const float* partials, int count,
+                                 long long stride, const void* weight, int weight_dtype,
+                                 const float* scale, float eps, int tokens, int hidden,
+                                 hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && hidden > 0, "norm_scale_add: bad sizes");
+  MK_REQUIRE(count >= 0 && (count == 0 || partials), "norm_scale_add: partial sums without a buffer");
+  MK_REQUIRE((y || count) && weight && h, "norm_scale_add: no operand");
+  MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "norm_scale_add: weight dtype %d",
+             weight_dtype);
+  if (tokens == 0) return 0;
+  const dim3 grid(tokens, std::max(1, std::min((hidden + 255) / 256, 512 / tokens)));
+  if (weight_dtype == MK_F32)
+    norm_scale_add_kernel<float><<<grid, 256, 0, stream>>>(h, y, partials, count, (size_t)stride,
+                                                              weight, scale, eps, hidden);
+  else
+    norm_scale_add_kernel<bf16_t><<<grid, 256, 0, stream>>>(h, y, partials, count, (size_t)stride,
+                                                               weight, scale, eps, hidden);
+  MK_LAUNCH_CHECK("norm_scale_add");
+  return 0;
+}
+
+extern "C" int mk_diff_heads(const void* a, void* out, int dtype, const float* gate,
+                             int gate_stride, float lambda, float eps, float out_scale, int tokens,
+                             int heads, int dv, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && heads > 0 && dv > 0, "diff_heads: bad sizes");
+  MK_REQUIRE(heads <= 65535, "diff_heads: too many heads (%d)", heads);
+  MK_REQUIRE(!gate || gate_stride >= heads, "diff_heads: gate rows of %d for %d heads", gate_stride, heads);
+  if (tokens == 0) return 0;
+  const dim3 grid(tokens, heads);
+  if (dtype == MK_F32)
+    diff_heads_kernel<float><<<grid, MK_WAVE, 0, stream>>>((const float*)a, (float*)out, gate,
+                                                             gate_stride, lambda, eps, out_scale, heads, dv);
+  else if (dtype == MK_BF16)
+    diff_heads_kernel<bf16_t><<<grid, MK_WAVE, 0, stream>>>((const bf16_t*)a, (bf16_t*)out, gate,
+                                                              gate_stride, lambda, eps, out_scale, heads, dv);
+  else
+    MK_REQUIRE(false, "diff_heads: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("diff_heads");
   return 0;
 }
 

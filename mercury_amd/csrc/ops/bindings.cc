@@ -39,7 +39,9 @@ py::bytes blob(const P& params) {
 }
 
 GateAct act_from(int kind, float limit, float alpha, float beta) {
-  if (kind != 0 && kind != 1) throw KernelError("unknown gate activation " + std::to_string(kind));
+  if (kind != MK_ACT_SILU && kind != MK_ACT_SWISH_CLAMP && kind != MK_ACT_GELU_TANH) {
+    throw KernelError("unknown gate activation " + std::to_string(kind));
+  }
   GateAct a;
   a.kind = kind;
   a.limit = limit;
@@ -242,6 +244,19 @@ void bind_ops(py::module_& m) {
     p.prep.temp_every = get<int>(d, "temp_every", 0);
     p.prep.values_are_keys = get<bool>(d, "values_are_keys", false) ? 1 : 0;
     p.prep.value_dim = get<int>(d, "value_dim", 0);
+    p.prep.maps = get<int>(d, "maps", 1);
+    p.head_gate = get<bool>(d, "head_gate", false) ? 1 : 0;
+    p.prep.extra_cols = p.head_gate ? p.qkv.n_q : 0;
+    p.keep_first = get<int>(d, "keep_first", 0);
+    p.diff_lambda = get<float>(d, "diff_lambda", 0.f);
+    p.diff_eps = get<float>(d, "diff_eps", 0.f);
+    p.diff_scale = get<float>(d, "diff_scale", 1.f);
+    if (p.prep.maps != 1 && p.prep.maps != 2) throw KernelError("attention: one or two maps a head");
+    if (p.prep.maps > 1 && p.qkv.head_dim % p.prep.maps) {
+      throw KernelError("attention: the maps of a head are equal parts of its key row");
+    }
+    if (p.head_gate && p.prep.maps == 1) throw KernelError("attention: a gate per head comes with two maps");
+    if (p.keep_first < 0) throw KernelError("attention: negative count of kept first keys");
     if ((p.prep.q_norm == nullptr) != (p.prep.k_norm == nullptr)) {
       throw KernelError("attention: a norm for queries and keys alike");
     }
@@ -293,6 +308,57 @@ void bind_ops(py::module_& m) {
     }
     return blob(p);
   });
+  m.def("retention_params", [](const py::kwargs& kw) {
+    const py::dict d = kw;
+    RetentionParams p;
+    RetentionArgs& a = p.args;
+    a.w_in = ptr_of<const void>(d, "w_in");
+    a.w_out = ptr_of<const void>(d, "w_out");
+    a.decay = ptr_of<const float>(d, "decay");
+    a.heads = get<int>(d, "heads", 0);
+    a.dim = get<int>(d, "dim", 0);
+    a.vdim = get<int>(d, "vdim", 0);
+    a.k_scale = get<float>(d, "k_scale", 1.f);
+    a.eps = get<float>(d, "eps", 0.f);
+    a.pos.rotary_dim = get<int>(d, "rotary_dim", 0);
+    a.pos.cos = ptr_of<const float>(d, "cos");
+    a.pos.sin = ptr_of<const float>(d, "sin");
+    a.pos.table_positions = get<int>(d, "table_positions", 0);
+    a.state = ptr_of<float>(d, "state");
+    a.slot_floats = get<long long>(d, "slot_floats", 0);
+    if (a.heads <= 0 || a.dim <= 0 || a.vdim <= 0 || a.pos.rotary_dim < 0 ||
+        a.pos.rotary_dim > a.dim || a.pos.rotary_dim % 2 ||
+        a.slot_floats < (long long)a.heads * a.dim * a.vdim) {
+      throw KernelError("retention: bad sizes");
+    }
+    if (get<bool>(d, "interleaved", false)) {
+      throw KernelError("retention: queries and keys turn in the half-split layout");
+    }
+    return blob(p);
+  });
+  m.def("post_norm_params", [](const std::string& kind_name, const py::bytes& sub, uintptr_t weight,
+                               int weight_dtype, uintptr_t scale, float eps) {
+    const OpKind& kind = OpRegistry::instance().get(kind_name);
+    if (kind.flags & MK_OP_FOLDS_PENDING) {
+      throw KernelError("the sublayer of a post norm cannot be an operation that adds up partial sums");
+    }
+    PostNormParams p;
+    p.eps = eps;
+    p.weight = as_ptr<const void>(weight);
+    p.weight_dtype = weight_dtype;
+    p.scale = as_ptr<const float>(scale);
+    p.run = kind.run;
+    p.tiles = kind.tiles;
+    p.flags = kind.flags;
+    std::string out(sizeof p, '\0');
+    out.resize((out.size() + 15) / 16 * 16, '\0');
+    p.offset = (int)out.size();
+    out += std::string(sub);
+    std::memcpy(&out[0], &p, sizeof p);
+    return py::bytes(out);
+  }, py::arg("kind"), py::arg("sublayer"), py::arg("weight"), py::arg("weight_dtype"),
+     py::arg("scale") = 0, py::arg("eps") = 0.f,
+     "The parameter block of a 'post_norm' operation around one sublayer (kind, parameter bytes).");
   m.def("normed_sum_params", [](float mult, float eps, int weight_dtype,
                                  const std::vector<std::tuple<std::string, py::bytes, uintptr_t>>& subs) {
     if (subs.empty() || (int)subs.size() > kNormedSumMax) {
@@ -394,8 +460,19 @@ void bind_ops(py::module_& m) {
     a.renormalize = get<bool>(d, "renormalize", false) ? 1 : 0;
     a.act = act_from(get<int>(d, "act", 0), get<float>(d, "limit", 0.f), get<float>(d, "alpha", 1.f),
                      get<float>(d, "beta", 0.f));
+    a.shared_gate_up = ptr_of<const void>(d, "shared_gate_up");
+    a.shared_down = ptr_of<const void>(d, "shared_down");
+    a.shared_gate = ptr_of<const void>(d, "shared_gate");
+    a.shared_ff = get<int>(d, "shared_ff", 0);
+    a.shared_act = act_from(get<int>(d, "shared_act", 0), get<float>(d, "shared_limit", 0.f),
+                            get<float>(d, "shared_alpha", 1.f), get<float>(d, "shared_beta", 0.f));
     if (a.experts <= 0 || a.top <= 0 || a.top > a.experts || a.ff <= 0) {
       throw KernelError("routed experts: bad sizes");
+    }
+    if ((a.shared_gate_up == nullptr) != (a.shared_down == nullptr) ||
+        (a.shared_gate_up != nullptr && a.shared_ff <= 0) ||
+        (a.shared_gate != nullptr && a.shared_gate_up == nullptr)) {
+      throw KernelError("routed experts: a shared expert has both its matrices and a width");
     }
     return blob(p);
   });

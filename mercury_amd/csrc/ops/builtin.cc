@@ -104,6 +104,9 @@ AttendArgs attend_args(const AttentionParams& p) {
   a.distance_slopes = p.distance_slopes;
   a.sinks = p.sinks;
   a.value_dim = p.prep.value_dim;
+  a.keep_first = p.keep_first;
+  // two maps a head: each is a query of its own over the same keys and values
+  if (p.prep.maps > 1) a.n_q = p.qkv.n_q * p.prep.maps;
   return a;
 }
 
@@ -118,6 +121,23 @@ int run_attention(const void* params, mk_op_context* ctx) {
     if (p.prep.active() && ctx->stream_fixed) {
       throw KernelError("attention: norms over q and k, a query temperature or values that are "
                         "keys do not run on a stream in fixed point");
+    }
+    if (p.prep.maps > 1 || p.head_gate) {
+      // maps combined, normed per head and gated between the attention and its projection
+      if (p.prep.maps != 1 && p.prep.maps != 2) throw KernelError("attention: one or two maps a head");
+      const float* raw = nullptr;
+      int raw_stride = 0;
+      const Queries q = qkv_prepared(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, p.prep, arrays,
+                                     &raw, &raw_stride);
+      const AttendArgs a = attend_args(p);
+      const void* attended = attend(l, q, a, arrays, s);
+      const float* gate = p.head_gate && raw ? raw + (raw_stride - p.prep.extra_cols) : nullptr;
+      if (p.prep.maps == 1) throw KernelError("attention: a gate per head comes with two maps");
+      const void* heads = diff_heads(l, attended, s.num_tokens, p.qkv.n_q, a.v_dim(), gate,
+                                     raw_stride, p.diff_lambda, p.diff_eps, p.diff_scale);
+      project_into_stream(l, heads, s.num_tokens, p.w_o, ctx->hidden, p.qkv.n_q * a.v_dim(), p.b_o,
+                          p.b_o_dtype, ctx->h, ctx->out_pending, ctx->out_pending_count);
+      return;
     }
     const Queries q = p.prep.active()
         ? qkv_prepared(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, p.prep, arrays)
@@ -137,7 +157,7 @@ int tiles_attention(const void* params, const mk_step_shape* shape, mk_tile_need
   view.max_kv_len = shape->max_kv_len;
   const AttentionPlan plan = plan_for(shape->dtype, attend_args(p), view);
   if (!plan.mfma) return 0;
-  out->group = p.qkv.n_q / p.qkv.n_kv;
+  out->group = p.qkv.n_q * (p.prep.maps > 1 ? p.prep.maps : 1) / p.qkv.n_kv;
   out->tile_rows = plan.tile_rows;
   return 1;
 }
@@ -198,8 +218,61 @@ int run_routed_experts(const void* params, mk_op_context* ctx) {
     const int m = ctx->step->num_tokens;
     if (ctx->x_rows != m) throw KernelError("the experts read an x of every token");
     Launch l(ctx);
-    routed_experts(l, ctx->x, m, ctx->hidden, p.experts, ctx->h);
+    routed_experts(l, ctx->x, m, ctx->hidden, p.experts, ctx->h, ctx->out_pending,
+                   ctx->out_pending_count);
   });
+}
+
+int run_retention(const void* params, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    const RetentionParams& p = *static_cast<const RetentionParams*>(params);
+    const mk_step_view& s = *ctx->step;
+    if (ctx->x_rows != s.num_tokens) throw KernelError("the mixer reads an x of every token");
+    Launch l(ctx);
+    retention(l, ctx->x, s.num_tokens, ctx->hidden, p.args, s, ctx->h, ctx->out_pending,
+              ctx->out_pending_count);
+  });
+}
+
+// The sublayer adds into a zeroed buffer in the stream's place; what it leaves as partial sums
+// is added to that buffer inside the kernel that norms, scales and adds.
+int run_post_norm(const void* params, mk_op_context* ctx) {
+  const PostNormParams& p = *static_cast<const PostNormParams*>(params);
+  const int tokens = ctx->step->num_tokens;
+  float* const h = ctx->h;
+  float* y = nullptr;
+  {
+    const int code = guarded(ctx, [&] {
+      Launch l(ctx);
+      y = zeros(l, (long long)tokens * ctx->hidden);
+    });
+    if (code) return code;
+  }
+  ctx->h = y;
+  ctx->out_x = nullptr;
+  ctx->out_x_rows = ctx->out_x_live = 0;
+  ctx->out_pending = nullptr;
+  ctx->out_pending_count = 0;
+  const int ran = p.run(static_cast<const char*>(params) + p.offset, ctx);
+  ctx->h = h;
+  if (ran) return ran;
+  const float* parts = ctx->out_pending;
+  const int count = ctx->out_pending_count;
+  ctx->out_x = nullptr;
+  ctx->out_x_rows = ctx->out_x_live = 0;
+  ctx->out_pending = nullptr;
+  ctx->out_pending_count = 0;
+  ctx->out_logits_ready = 0;
+  return guarded(ctx, [&] {
+    Launch l(ctx);
+    norm_scale_add(l, h, y, parts, count, p.weight, p.weight_dtype, p.scale, p.eps, tokens,
+                   ctx->hidden);
+  });
+}
+
+int tiles_post_norm(const void* params, const mk_step_shape* shape, mk_tile_need* out) {
+  const PostNormParams& p = *static_cast<const PostNormParams*>(params);
+  return p.tiles ? p.tiles(static_cast<const char*>(params) + p.offset, shape, out) : 0;
 }
 
 int run_unary_mlp(const void* params, mk_op_context* ctx) {
@@ -408,6 +481,8 @@ void register_builtin_ops() {
   r.add(OpKind{"unary_mlp", &run_unary_mlp, nullptr, MK_OP_READS_X});
   r.add(OpKind{"state_space", &run_state_space, nullptr, MK_OP_READS_X});
   r.add(OpKind{"normed_sum", &run_normed_sum, &tiles_normed_sum, MK_OP_READS_X});
+  r.add(OpKind{"retention", &run_retention, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"post_norm", &run_post_norm, &tiles_post_norm, MK_OP_READS_X});
   r.add(OpKind{"keep_stream", &run_keep_stream, nullptr, MK_OP_KEPT_STREAM | MK_OP_FOLDS_PENDING});
   r.add(OpKind{"stream_mix", &run_stream_mix, nullptr, MK_OP_KEPT_STREAM | MK_OP_FOLDS_PENDING});
   r.add(OpKind{"head", &run_head, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});

@@ -37,6 +37,34 @@ struct AttentionParams {
   const float* distance_slopes = nullptr;   // [n_q]: slope * distance is subtracted from it
   const float* sinks = nullptr;             // [n_q]: exp(sink) once more in the denominator
   QkPrep prep;                              // norms over q and k, query temperature, v = k
+  int keep_first = 0;                       // with a window: the first keys stay visible past it
+  // Differential attention (prep.maps == 2): every head has two score maps over the same
+  // values; o = a1 - lambda a2, divided by its root mean square over the head (eps), times
+  // out_scale.  head_gate: the stacked projection ends in one gate column per head, and the
+  // head's output is multiplied by its sigmoid (with or without two maps).
+  float diff_lambda = 0.f, diff_eps = 0.f, diff_scale = 1.f;
+  int head_gate = 0;
+};
+
+// "retention": a decayed outer-product state per head and request (launch.h), its output
+// projection into h (or left as partial sums).
+struct RetentionParams {
+  RetentionArgs args;
+};
+
+// "post_norm": one sublayer whose output is RMS-normed over the model width and multiplied,
+// channel by channel, by a stored vector before it enters the stream:
+// h += scale .* (rmsnorm(f(x)) * weight).  Laid out as "parallel": this header, then the
+// sublayer's parameter block at `offset`.
+struct PostNormParams {
+  float eps = 0.f;
+  int weight_dtype = 0;
+  const void* weight = nullptr;
+  const float* scale = nullptr;     // float32 [hidden], or null
+  mk_op_run_fn run = nullptr;
+  mk_op_tiles_fn tiles = nullptr;
+  int flags = 0;
+  int offset = 0;
 };
 
 // "unary_mlp": h += act(x Wu^T) Wd^T for an activation of one operand (or left as partial sums).

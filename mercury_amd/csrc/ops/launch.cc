@@ -241,14 +241,18 @@ Queries qkv_project(Launch& l, const void* x, int m, int k, const QkvArgs& a, co
 }
 
 Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, const QkPrep& prep,
-                     const StepArrays& s) {
+                     const StepArrays& s, const float** raw, int* raw_stride) {
   const int d = a.head_dim, dv = prep.value_dim > 0 ? prep.value_dim : d;
   const int heads_kv = kv_heads(a);
-  const int width = a.n_q * d + heads_kv * d + (prep.values_are_keys ? 0 : heads_kv * dv);
+  const int maps = prep.maps > 1 ? prep.maps : 1;
+  const int width = a.n_q * d + heads_kv * d + (prep.values_are_keys ? 0 : heads_kv * dv) +
+                    prep.extra_cols;
   const float* qkv = (const float*)linear(l, x, m, a.w, width, k, a.bias,
                                           a.bias ? a.bias_dtype : kF32, nullptr, kF32, false);
-  void* q = l.alloc((size_t)m * a.n_q * d * l.elem());
-  if (l.dry() || m == 0) return {q, a.n_q * d};
+  if (raw) *raw = qkv;
+  if (raw_stride) *raw_stride = width;
+  void* q = l.alloc((size_t)m * a.n_q * maps * d * l.elem());
+  if (l.dry() || m == 0) return {q, a.n_q * maps * d};
   const PositionDesc& p = a.pos;
   check_core(need_core().mk_qk_prepare(
                  qkv, width, q, l.dtype(), prep.q_norm, prep.k_norm, prep.norm_dtype, prep.eps,
@@ -256,8 +260,8 @@ Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, c
                  p.interleaved ? 1 : 0, s.positions, s.token_seq, s.table, s.table_stride,
                  a.writes ? a.k_cache : nullptr, a.writes ? a.v_cache : nullptr,
                  a.writes ? a.page_size : 1, a.n_q, heads_kv, d, dv, prep.values_are_keys,
-                 a.writes ? 1 : 0, m, l.stream()), "qk_prepare");
-  return {q, a.n_q * d};
+                 a.writes ? 1 : 0, maps, m, l.stream()), "qk_prepare");
+  return {q, a.n_q * maps * d};
 }
 
 AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
@@ -271,6 +275,12 @@ AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
   if (a.v_dim() != a.head_dim) {
     if (force.kernel == 2) {
       throw KernelError("attention: the matrix-core kernels keep values as wide as keys");
+    }
+    return AttentionPlan();
+  }
+  if (a.window > 0 && a.keep_first > 0) {
+    if (force.kernel == 2) {
+      throw KernelError("attention: the matrix-core kernels keep no first keys past a window");
     }
     return AttentionPlan();
   }
@@ -310,8 +320,8 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
       check_core(need_core().mk_attention_generic_kv(
                      q.q, q.stride, out, a.n_q * a.v_dim(), a.k_cache, a.v_cache, l.dtype(),
                      s.positions, s.token_seq, s.table, s.table_stride, a.page_size, a.n_q, a.n_kv,
-                     d, a.v_dim(), a.scale, a.window, a.score_cap, a.distance_slopes, a.sinks, m,
-                     l.stream()), "attention");
+                     d, a.v_dim(), a.scale, a.window, a.window > 0 ? a.keep_first : 0, a.score_cap,
+                     a.distance_slopes, a.sinks, m, l.stream()), "attention");
     }
     return out;
   }
@@ -418,6 +428,48 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
   }
   check_mfma(t.mk_attention_out(part_o, part_ml, written, w_o, out, h_fixed, m, hidden, a.n_q, a.n_kv, d,
                                 heads_per_slice, wide ? 1 : 0, l.stream()), "attention_out");
+}
+
+void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float* gate,
+                 int gate_stride, float lambda, float eps, float out_scale) {
+  void* out = l.alloc((size_t)m * heads * dv * l.elem());
+  if (l.dry() || m == 0) return out;
+  check_core(need_core().mk_diff_heads(a, out, l.dtype(), gate, gate_stride, lambda, eps, out_scale,
+                                       m, heads, dv, l.stream()), "diff_heads");
+  return out;
+}
+
+void norm_scale_add(Launch& l, float* h, const float* y, const float* partials, int count,
+                    const void* weight, int weight_dtype, const float* scale, float eps,
+                    int tokens, int hidden) {
+  if (l.dry() || tokens == 0) return;
+  check_core(need_core().mk_norm_scale_add(h, y, partials, count, (long long)tokens * hidden,
+                                           weight, weight_dtype, scale, eps, tokens, hidden,
+                                           l.stream()), "norm_scale_add");
+}
+
+void retention(Launch& l, const void* x, int m, int hidden, const RetentionArgs& a,
+               const mk_step_view& step, float* h, const float*& pending, int& pending_count) {
+  pending = nullptr;
+  pending_count = 0;
+  const int width = a.in_width(), qk = a.heads * a.dim, inner = a.heads * a.vdim;
+  const float* proj = (const float*)linear(l, x, m, a.w_in, width, hidden, nullptr, kF32, nullptr,
+                                           kF32, false);
+  float* y = (float*)l.alloc((size_t)m * inner * 4);
+  void* normed = l.alloc((size_t)m * inner * l.elem());
+  if (!l.dry() && m > 0) {
+    const KernelTable& t = need_core();
+    if (!a.state) throw KernelError("retention: no state tensor");
+    check_core(t.mk_retention_scan(proj, width, 0, qk, 2 * qk, a.decay, a.k_scale, a.pos.cos,
+                                   a.pos.sin, a.pos.table_positions, a.pos.rotary_dim,
+                                   step.positions, step.cu_q, step.state_slots, a.state,
+                                   a.slot_floats, a.heads, a.dim, a.vdim, y, m, step.num_seqs,
+                                   l.stream()), "retention_scan");
+    check_core(t.mk_head_norm_gate(y, normed, l.dtype(), proj + 2 * qk + inner, width, a.eps, m,
+                                   a.heads, a.vdim, l.stream()), "head_norm_gate");
+  }
+  project_into_stream(l, normed, m, a.w_out, hidden, inner, nullptr, kF32, h, pending,
+                      pending_count);
 }
 
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
@@ -637,7 +689,7 @@ void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scal
       check_core(need_core().mk_attention_generic_kv(
                      q.q, q.stride, out, a.heads * dv, a.k_cache, a.v_cache, l.dtype(), s.positions,
                      s.token_seq, s.table, s.table_stride, a.page_size, a.heads, 1, dk, dv, scale,
-                     0, 0.f, nullptr, nullptr, m, l.stream()), "latent_attention");
+                     0, 0, 0.f, nullptr, nullptr, m, l.stream()), "latent_attention");
     }
     return out;
   }
@@ -661,7 +713,27 @@ void* latent_values(Launch& l, const void* summed, int m, const LatentArgs& a) {
                          a.vdim, a.kv_rank, nullptr, 0, 0);
 }
 
-void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y) {
+namespace {
+// The shared expert beside the routed ones: a gated feed-forward of every token, its
+// activations times the token's gate, its down-projection into the same sum.
+void shared_expert(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y,
+                   const float*& pending, int& pending_count) {
+  if (!a.shared_gate_up) return;
+  void* act = gated(l, x, m, hidden, a.shared_gate_up, a.shared_ff, -2, nullptr, a.shared_act);
+  if (a.shared_gate && !l.dry() && m > 0) {
+    check_core(need_core().mk_row_gate(act, x, a.shared_gate, l.dtype(), m, a.shared_ff, hidden,
+                                       l.stream()), "row_gate");
+  }
+  project_into_stream(l, act, m, a.shared_down, hidden, a.shared_ff, nullptr, kF32, y, pending,
+                      pending_count);
+}
+}  // namespace
+
+void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y,
+                    const float*& pending, int& pending_count) {
+  pending = nullptr;
+  pending_count = 0;
+  shared_expert(l, x, m, hidden, a, y, pending, pending_count);
   const float* logits = (const float*)linear(l, x, m, a.w_router, a.experts, hidden, nullptr, kF32,
                                              nullptr, kF32, false);
   int* ids = (int*)l.alloc((size_t)m * a.top * 4);

@@ -150,14 +150,23 @@ struct QkPrep {
   int temp_every = 0;
   int values_are_keys = 0;
   int value_dim = 0;            // 0: as wide as the keys
+  // A head of `maps` score maps side by side (each turned by itself): the queries come back
+  // as n_q * maps rows a key row wide, every one zero outside its own map.
+  int maps = 1;
+  // Further columns of the stacked projection behind q, k, v that belong to the caller (a
+  // gate's logits): projected in the same product, left alone here.
+  int extra_cols = 0;
   bool active() const {
-    return q_norm != nullptr || temp_every > 0 || values_are_keys != 0 || value_dim > 0;
+    return q_norm != nullptr || temp_every > 0 || values_are_keys != 0 || value_dim > 0 ||
+           maps > 1 || extra_cols > 0;
   }
 };
 // qkv_project for such an attention: the projection in float32, then one kernel for all of
 // the above, the rotation and the cache write.
+// `raw`, when not null, receives the float32 projection and `raw_stride` its row width (the
+// extra columns start behind q, k and v).
 Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, const QkPrep& prep,
-                     const StepArrays& s);
+                     const StepArrays& s, const float** raw = nullptr, int* raw_stride = nullptr);
 
 // Rotation and cache write of an already projected qkv [m, row_stride] (q rotated in place).
 void rope_kv_write(Launch& l, void* qkv, int row_stride, int m, const QkvArgs& a,
@@ -170,6 +179,7 @@ void* qkv_finish(Launch& l, const float* parts, int slices, int m, const QkvArgs
 
 struct AttendArgs {
   int n_q = 0, n_kv = 0, head_dim = 0, page_size = 0, window = 0;
+  int keep_first = 0;    // with a window: the sequence's first keys stay visible past it
   int value_dim = 0;     // 0: values as wide as keys
   int v_dim() const { return value_dim > 0 ? value_dim : head_dim; }
   float scale = 0.f;
@@ -209,6 +219,34 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
                         const mk_step_view& step, const void* w_o, const void* b_o, int b_o_dtype,
                         int hidden, float* h, const float*& pending, int& pending_count,
                         AttendForce force = {}, int fold = -1, long long* h_fixed = nullptr);
+
+// Two maps per head combined: a [m, heads, 2, dv] -> [m, heads dv] in the compute dtype,
+// (a1 - lambda a2) / rms * out_scale * sigmoid(gate) (see mk_diff_heads).
+void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float* gate,
+                 int gate_stride, float lambda, float eps, float out_scale);
+
+// h += scale .* (rmsnorm(y + its partial sums) * weight) (see mk_norm_scale_add).
+void norm_scale_add(Launch& l, float* h, const float* y, const float* partials, int count,
+                    const void* weight, int weight_dtype, const float* scale, float eps,
+                    int tokens, int hidden);
+
+// Retention: one projection [q | k | v | gate] in float32, the decayed recurrence per head from
+// the state earlier steps left (queries and keys turned, keys scaled), a norm per head, the
+// gate silu(gate columns), the output projection into h.  `state` holds [heads, dim, vdim]
+// floats per slot.
+struct RetentionArgs {
+  const void* w_in = nullptr;      // [2 heads dim + 2 heads vdim, hidden]
+  const void* w_out = nullptr;     // [hidden, heads vdim]
+  const float* decay = nullptr;    // [heads]
+  int heads = 0, dim = 0, vdim = 0;
+  float k_scale = 1.f, eps = 0.f;
+  PositionDesc pos;
+  float* state = nullptr;
+  long long slot_floats = 0;
+  int in_width() const { return 2 * heads * dim + 2 * heads * vdim; }
+};
+void retention(Launch& l, const void* x, int m, int hidden, const RetentionArgs& a,
+               const mk_step_view& step, float* h, const float*& pending, int& pending_count);
 
 // act = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, k].  tile_config: -2 by the
 // sizes, else the tiled kernel with that configuration (-1: its own choice).
@@ -315,7 +353,15 @@ struct ExpertArgs {
   float scale = 1.f;
   int renormalize = 0;
   GateAct act;
+  // A shared expert every token runs, added beside the chosen ones (null: none): a gated
+  // feed-forward [2 shared_ff, hidden] / [hidden, shared_ff] with an activation of its own,
+  // multiplied by sigmoid(x . shared_gate) when shared_gate [hidden] is there.
+  const void *shared_gate_up = nullptr, *shared_down = nullptr, *shared_gate = nullptr;
+  int shared_ff = 0;
+  GateAct shared_act;
 };
-void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y);
+// The shared expert's down-projection goes into y or is left as partial sums (pending).
+void routed_experts(Launch& l, const void* x, int m, int hidden, const ExpertArgs& a, float* y,
+                    const float*& pending, int& pending_count);
 
 }  // namespace mercury

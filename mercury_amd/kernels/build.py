@@ -35,6 +35,7 @@ LIBRARIES = {
         "experts.hip",
         "mixers.hip",
         "state_space.hip",
+        "retention.hip",
         "sampling.hip",
         "random_fill.hip",
     ],

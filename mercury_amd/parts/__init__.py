@@ -3,7 +3,7 @@
 from .attention import Attention
 from .base import (CacheSpec, FeedForward, LayerCache, Mixer, Norm, Part, PositionDescriptor,
                    PositionEncoding, StateSpec, TensorSpec)
-from .block import ParallelBlock, PreNormBlock
+from .block import ParallelBlock, PreNormBlock, PrePostNormBlock
 from .embedding import OutputHead, TokenEmbedding
 from .experts import RoutedExperts
 from .feedforward import GatedMLP, UnaryMLP
@@ -15,6 +15,7 @@ from .norm import RMSNorm
 from .position import NoPosition, RotaryPosition
 from .state_space import StateSpaceMixer
 from .stream_mix import StreamMix
+from .retention import Retention
 from .registry import (build_part, known, register_block, register_ffn, register_mixer,
                        register_norm, register_position)
 
@@ -25,16 +26,18 @@ register_ffn("routed_experts")(RoutedExperts)
 register_ffn("unary_mlp")(UnaryMLP)
 register_mixer("state_space")(StateSpaceMixer)
 register_mixer("normed_sum")(NormedMixerSum)
+register_mixer("retention")(Retention)
 register_norm("rmsnorm")(RMSNorm)
 register_position("rotary")(RotaryPosition)
 register_position("none")(NoPosition)
 register_block("pre_norm")(PreNormBlock)
 register_block("parallel")(ParallelBlock)
+register_block("pre_post_norm")(PrePostNormBlock)
 
 __all__ = [
     "Attention", "CacheSpec", "CallerStep", "DecoderModel", "FeedForward", "GatedMLP",
     "LatentAttention", "LayerCache", "LayerCall", "Mixer", "NoPosition", "Norm", "OneOp", "OutputHead", "Part",
-    "ParallelBlock", "PositionDescriptor", "PositionEncoding", "PreNormBlock", "Registers",
+    "ParallelBlock", "PositionDescriptor", "PrePostNormBlock", "Retention", "PositionEncoding", "PreNormBlock", "Registers",
     "RoutedExperts", "NormedMixerSum", "StateSpaceMixer", "StreamMix", "UnaryMLP",
     "RMSNorm", "RotaryPosition", "StateSpec", "TensorSpec", "TokenEmbedding", "build_part", "known",
     "register_block", "register_ffn", "register_mixer", "register_norm", "register_position",

@@ -12,7 +12,8 @@ from .lowering import OneOp
 # Leaf names of the stored tensors, under the prefix the builder gives; an architecture whose
 # checkpoints call them otherwise passes its own map.
 DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj",
-                 "q_norm": "q_norm", "k_norm": "k_norm", "sink": "sink"}
+                 "q_norm": "q_norm", "k_norm": "k_norm", "sink": "sink", "gate": "g_proj",
+                 "lq1": "lambda_q1", "lk1": "lambda_k1", "lq2": "lambda_q2", "lk2": "lambda_k2"}
 
 
 class Attention(Mixer):
@@ -39,6 +40,21 @@ class Attention(Mixer):
     `sinks`: a stored number per query head (``<sink>.weight`` [n_q]) whose exponential stands
     once more in the softmax's denominator, unscaled, with no key or value behind it.
     `k_bias` / `v_bias` (default: as `qkv_bias`) say which of the projections have a bias.
+    `keep_first` (with a `window`): the sequence's first `keep_first` keys stay visible to
+    queries whose window has passed them, at their true positions.  `cache_window` /
+    `cache_keep_first` widen what the cache keeps beyond this layer's own mask, for a slot that
+    layers with other masks read.
+    `maps=2`: differential attention.  `head_dim` is a head's whole key row, two score maps of
+    head_dim / 2 dims side by side in the q and k projections (each map turned by itself over
+    its first dims; `position` is built for a map's width); both maps are softmax attentions
+    over the same values, combined as  o = a1 - lam * a2,
+    lam = exp(<lq1, lk1>) - exp(<lq2, lk2>) + `diff_init`  (four stored vectors of a map's
+    width, one number for the layer), then o / rms(o) over the head (eps `norm_eps`, no weight)
+    times 1 - `diff_init`.  `head_gate`: a projection ``<gate>.weight`` [n_q, hidden] of the
+    mixer's input gives one number a head, whose sigmoid multiplies the head's output before
+    the output projection.
+    `own_kv=False`: the layer has no key and value projections; it reads a cache slot that
+    another layer writes (whose head counts, widths and rotation are its own).
     """
 
     graph_safe = True   # forward launches kernels only: a decode step may be captured in a graph
@@ -49,7 +65,10 @@ class Attention(Mixer):
                  names: dict | None = None, score_cap: float | None = None,
                  values: str = "projected", value_dim: int | None = None,
                  qk_norm: str | None = None, norm_eps: float = 1e-6,
-                 q_temp: tuple | None = None, sinks: bool = False):
+                 q_temp: tuple | None = None, sinks: bool = False, keep_first: int = 0,
+                 maps: int = 1, diff_init: float = 0.0, head_gate: bool = False,
+                 cache_window: int | None = -1, cache_keep_first: int | None = None,
+                 own_kv: bool = True):
         if n_q % n_kv:
             raise ValueError(f"{n_q} query heads are not a multiple of {n_kv} key/value heads")
         self.hidden, self.n_q, self.n_kv, self.head_dim = int(hidden), int(n_q), int(n_kv), int(head_dim)
@@ -71,6 +90,25 @@ class Attention(Mixer):
         if self.q_temp and self.q_temp[1] <= 0:
             raise ValueError("the query temperature's period must be positive")
         self.sinks = bool(sinks)
+        self.keep_first = int(keep_first) if self.window else 0
+        if self.keep_first < 0:
+            raise ValueError("a window keeps no negative number of first keys")
+        self.maps, self.diff_init, self.head_gate = int(maps), float(diff_init), bool(head_gate)
+        if self.maps not in (1, 2) or self.head_dim % self.maps:
+            raise ValueError(f"{maps} maps in a key row of {head_dim}: one, or two equal halves")
+        if self.head_gate and self.maps == 1:
+            raise ValueError("a gate per head comes with two maps a head")
+        if self.maps > 1 and (self.qkv_bias or self.score_cap or self.sinks or self.qk_norm
+                              or self.q_temp or self.values_are_keys):
+            raise ValueError("two maps a head go with plain projections and a plain softmax")
+        # what the cache slot keeps: this layer's own mask unless told otherwise
+        self.cache_window = self.window if cache_window == -1 else (int(cache_window) if cache_window else None)
+        self.cache_keep_first = self.keep_first if cache_keep_first is None else int(cache_keep_first)
+        self.diff_lambda = 0.0
+        self.w_q_gate = None
+        self.own_kv = bool(own_kv)
+        if not self.own_kv and self.values_are_keys:
+            raise ValueError("values that are keys are a layer's own")
         self.names = {**DEFAULT_NAMES, **(names or {})}
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
         self.w_q_norm = self.w_k_norm = self.sink = None
@@ -81,17 +119,21 @@ class Attention(Mixer):
         """Whether q and k get more than a rotation between projection and cache (the kernels
         then take the projection in float32 and do all of it in one pass)."""
         return bool(self.values_are_keys or self.qk_norm or self.q_temp
-                    or self.value_dim != self.head_dim)
+                    or self.value_dim != self.head_dim or self.maps > 1)
 
     # ---- declarations
 
     def cache_spec(self) -> CacheSpec:
         value_dim = None if self.value_dim == self.head_dim else self.value_dim
-        return CacheSpec(self.n_kv, self.head_dim, self.window, value_dim)
+        return CacheSpec(self.n_kv, self.head_dim, self.cache_window, value_dim,
+                         keep_first=self.cache_keep_first if self.cache_window else 0)
 
     def _projections(self) -> list:
         """The stacked projections in order: (name key, rows)."""
-        out = [("q", self.n_q * self.head_dim), ("k", self.n_kv * self.head_dim)]
+        out = [("q", self.n_q * self.head_dim)]
+        if not self.own_kv:
+            return out
+        out.append(("k", self.n_kv * self.head_dim))
         if not self.values_are_keys:
             out.append(("v", self.n_kv * self.value_dim))
         return out
@@ -113,13 +155,29 @@ class Attention(Mixer):
                                                         init="one_plus_normal")
         if self.sinks:
             specs[f"{n['sink']}.weight"] = TensorSpec((self.n_q,), role="vector")
+        if self.maps > 1:
+            for key in ("lq1", "lk1", "lq2", "lk2"):
+                specs[n[key]] = TensorSpec((self.head_dim // self.maps,), role="vector")
+        if self.head_gate:
+            specs[f"{n['gate']}.weight"] = TensorSpec((self.n_q, h))
         return specs
 
     def bind(self, params, dtype, device) -> None:
         n = self.names
         # One projection for q, k and v: rows [q heads | k heads | v heads].
         keys = [key for key, _rows in self._projections()]
-        self.w_qkv = torch.cat([params[f"{n[key]}.weight"] for key in keys], dim=0).contiguous()
+        stacked = [params[f"{n[key]}.weight"] for key in keys]
+        if self.head_gate:
+            # the gate's rows ride behind q, k, v in the same product; a layer that reads
+            # another's keys and values projects [q | gate] only
+            gate = params[f"{n['gate']}.weight"]
+            stacked.append(gate)
+            self.w_q_gate = torch.cat([stacked[0], gate], dim=0).contiguous()
+        self.w_qkv = torch.cat(stacked, dim=0).contiguous()
+        if self.maps > 1:
+            dot = lambda a, b: (params[n[a]].float() * params[n[b]].float()).sum()
+            self.diff_lambda = float(torch.exp(dot("lq1", "lk1")) - torch.exp(dot("lq2", "lk2"))
+                                     + self.diff_init)
         if self.qkv_bias:
             biases = [params[f"{n[key]}.bias"] for key in keys]
             common = torch.float32 if any(b.dtype == torch.float32 for b in biases) else dtype
@@ -140,7 +198,7 @@ class Attention(Mixer):
     def weight_bytes(self) -> int:
         total = 0
         for t in (self.w_qkv, self.b_qkv, self.w_o, self.b_o, self.w_q_norm, self.w_k_norm,
-                  self.sink):
+                  self.sink):   # (w_q_gate repeats rows of w_qkv)
             if t is not None:
                 total += t.numel() * t.element_size()
         return total
@@ -162,10 +220,15 @@ class Attention(Mixer):
         bias_code = lambda t: ops.dtype_code(t.dtype) if t is not None else ops.F32
         ptr = lambda t: 0 if t is None else t.data_ptr()
         w, b = self.w_qkv, self.b_qkv
-        if not cache.writes:
+        if cache.writes and not self.own_kv:
+            raise ValueError("an attention without key and value projections reads a cache "
+                             "another layer writes")
+        if not cache.writes and self.own_kv:
             # Reads a cache another entry fills: only the queries are projected.
             rows = self.n_q * self.head_dim
             w, b = w[:rows], None if b is None else b[:rows]
+            if self.head_gate:
+                w = self.w_q_gate
         # (a kind of its own where the fixed-point stream's kernels would not do the same)
         program.append("attention_prepared" if self.prepared or self.sinks else "attention",
                        core.attention_params(
@@ -182,7 +245,10 @@ class Attention(Mixer):
             norm_eps=self.norm_eps, temp_coef=self.q_temp[0] if self.q_temp else 0.0,
             temp_every=self.q_temp[1] if self.q_temp else 0,
             values_are_keys=self.values_are_keys,
-            value_dim=self.value_dim if self.prepared else 0))
+            value_dim=self.value_dim if self.prepared else 0,
+            keep_first=self.keep_first, maps=self.maps, head_gate=self.head_gate,
+            diff_lambda=self.diff_lambda, diff_eps=self.norm_eps,
+            diff_scale=1.0 - self.diff_init if self.maps > 1 else 1.0))
 
     def forward(self, x, step, cache, state, accum):
         if self.position.describe() is not None:

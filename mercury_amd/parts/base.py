@@ -72,23 +72,26 @@ class TensorSpec:
 class CacheSpec:
     """Per-token cache need of a mixer: keys of `kv_heads` heads of `head_dim` and values of as
     many heads of `value_dim` (default: the keys' width), stored as `dtype` (default: the
-    model's compute dtype); all earlier tokens (`window` None) or the last `window` of them."""
+    model's compute dtype); all earlier tokens (`window` None) or the last `window` of them,
+    beside which the sequence's first `keep_first` tokens stay."""
 
     kv_heads: int
     head_dim: int
     window: int | None = None
     value_dim: int | None = None
     dtype: torch.dtype | None = None
+    keep_first: int = 0
 
     @property
     def v_dim(self) -> int:
         return self.head_dim if self.value_dim is None else self.value_dim
 
     def as_tuple(self) -> tuple:
-        """(kv_heads, key width, value width, dtype code or -1, window or 0): what the cache
-        manager groups slots by."""
+        """(kv_heads, key width, value width, dtype code or -1, window or 0, first tokens a
+        window keeps): what the cache manager groups slots by."""
         code = -1 if self.dtype is None else {torch.float32: 0, torch.bfloat16: 1}[self.dtype]
-        return (self.kv_heads, self.head_dim, self.v_dim, code, self.window or 0)
+        return (self.kv_heads, self.head_dim, self.v_dim, code, self.window or 0,
+                self.keep_first if self.window else 0)
 
 
 @dataclass(frozen=True)

@@ -83,6 +83,119 @@ class PreNormBlock(Part):
         return pending
 
 
+class PrePostNormBlock(Part):
+    """A norm before and after each sublayer, and a stored vector per channel on what enters
+    the stream:
+
+        h += scale_1 * post_1(mixer(norm_1(h)));   h += scale_2 * post_2(ffn(norm_2(h)))
+
+    with h the float32 residual stream, every norm an :class:`RMSNorm` over the model width
+    and scale_i ``<names["scale_mixer"]>`` / ``<names["scale_ffn"]>`` (float32 [hidden]; absent
+    when `layer_scale` is off).  `ffn` may be None.  Lowered, a sublayer is its norm and one
+    ``post_norm`` operation that holds the sublayer's own operation and runs it over a zeroed
+    buffer in the stream's place.  `names` gives the stored sub-prefix of every part:
+    ``{"mixer", "ffn", "norm_mixer", "norm_ffn", "post_mixer", "post_ffn", "scale_mixer",
+    "scale_ffn"}``.
+    """
+
+    def __init__(self, mixer: Mixer, ffn: FeedForward | None, norm_mixer: Norm,
+                 norm_ffn: Norm | None, post_mixer: Norm, post_ffn: Norm | None, names: dict,
+                 layer_scale: bool = True):
+        self.mixer, self.ffn = mixer, ffn
+        self.norm_mixer, self.norm_ffn = norm_mixer, norm_ffn
+        self.post_mixer, self.post_ffn = post_mixer, post_ffn
+        self.layer_scale = bool(layer_scale)
+        self.names = dict(names)
+        self.scale_mixer = self.scale_ffn = None
+        self._alone: dict = {}
+
+    def _children(self):
+        out = [("mixer", self.mixer), ("norm_mixer", self.norm_mixer), ("post_mixer", self.post_mixer)]
+        if self.ffn is not None:
+            out += [("ffn", self.ffn), ("norm_ffn", self.norm_ffn), ("post_ffn", self.post_ffn)]
+        return out
+
+    def _scales(self):
+        if not self.layer_scale:
+            return []
+        return ["scale_mixer"] + (["scale_ffn"] if self.ffn is not None else [])
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for _, part in self._children())
+
+    def lowerable_with(self, state) -> bool:
+        if state is not None and not getattr(self.mixer, "lowers_state", False):
+            return False
+        return all(part.can_lower() for _, part in self._children())
+
+    def _wrapped(self, program, sub: "_Recorder", post: Norm, scale) -> None:
+        if len(sub.ops) != 1:
+            raise ValueError("a sublayer between two norms lowers itself to one operation")
+        if getattr(post, "one_plus", False) and post.weight is None:
+            raise ValueError("the norm behind a sublayer has no weight yet")
+        program.append("post_norm", core.post_norm_params(
+            sub.ops[0][0], sub.ops[0][1], post.weight.data_ptr(), ops.dtype_code(post.weight.dtype),
+            0 if scale is None else scale.data_ptr(), post.eps))
+
+    def lower(self, program, cache, state=None) -> None:
+        self.norm_mixer.lower(program)
+        sub = _Recorder()
+        if state is None:
+            self.mixer.lower(sub, cache)
+        else:
+            self.mixer.lower(sub, cache, state)
+        self._wrapped(program, sub, self.post_mixer, self.scale_mixer)
+        if self.ffn is not None:
+            self.norm_ffn.lower(program)
+            sub = _Recorder()
+            self.ffn.lower(sub)
+            self._wrapped(program, sub, self.post_ffn, self.scale_ffn)
+
+    def param_specs(self) -> dict:
+        from .base import TensorSpec
+
+        specs = {}
+        for key, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[self.names[key] + name] = spec
+        width = self.post_mixer.size
+        for key in self._scales():
+            specs[self.names[key]] = TensorSpec((width,), role="vector", init="one_plus_normal")
+        return specs
+
+    def bind(self, params, dtype, device) -> None:
+        scale_names = {self.names[key] for key in self._scales()}
+        for key, part in self._children():
+            prefix = self.names[key]
+            part.bind({n[len(prefix):]: t for n, t in params.items()
+                       if n.startswith(prefix) and n not in scale_names}, dtype, device)
+        if self.layer_scale:
+            self.scale_mixer = params[self.names["scale_mixer"]].float().contiguous()
+            if self.ffn is not None:
+                self.scale_ffn = params[self.names["scale_ffn"]].float().contiguous()
+        self._alone.clear()
+
+    def prepare(self, max_positions: int, device) -> None:
+        self.mixer.prepare(max_positions, device)
+
+    def weight_bytes(self) -> int:
+        total = sum(part.weight_bytes() for _, part in self._children())
+        return total + sum(t.numel() * 4 for t in (self.scale_mixer, self.scale_ffn) if t is not None)
+
+    def forward(self, h, step, cache, state, dtype, pending=None):
+        if not self.lowerable_with(state):
+            raise NotImplementedError("a layer with norms behind its sublayers runs as operations "
+                                      "of the host core: every part of it must lower itself")
+        key = (None if cache is None else cache.k.data_ptr(), None if state is None else state.data_ptr())
+        alone = self._alone.get(key)
+        if alone is None:
+            alone = self._alone[key] = OneOp(dtype, h.shape[1], 0,
+                                             lambda program: self.lower(program, cache, state))
+        _logits, _x, left = alone.run(step, h, pending=pending)
+        return left
+
+
 class _Recorder:
     """Stands in for a program while a sublayer lowers itself: keeps what it appends."""
 

@@ -8,9 +8,9 @@ from ..hostcore import core
 from .base import FeedForward, TensorSpec
 from .lowering import OneOp
 
-ACTIVATIONS = ("silu", "swish_clamp")
+ACTIVATIONS = ("silu", "swish_clamp", "gelu_tanh")
 # the kernels' codes of the activations
-ACTIVATION_CODES = {"silu": 0, "swish_clamp": 1}
+ACTIVATION_CODES = {"silu": 0, "swish_clamp": 1, "gelu_tanh": 2}
 DEFAULT_NAMES = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
 
 
@@ -20,6 +20,7 @@ class GatedMLP(FeedForward):
     ``"silu"``: silu(g) * u (reference: mercury/model/qwen2.py:34-42).
     ``"swish_clamp"``: g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit) and
     u' = clamp(u, -limit, limit).
+    ``"gelu_tanh"``: 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u.
 
     `names` maps gate, up, down to the stored tensors' leaf names (default ``gate_proj``,
     ``up_proj``, ``down_proj``)."""
