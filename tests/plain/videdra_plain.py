@@ -36,6 +36,23 @@ def load_folder(folder, dtype=torch.float32):
     return config, tensors
 
 
+def to_bf16(t):
+    """What a tensor is after a round trip through bfloat16."""
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
+def same(t):
+    return t
+
+
+def read_config(folder) -> dict:
+    return json.loads((Path(folder) / "config.json").read_text())
+
+
+def read_weights(folder, dtype=torch.float32) -> dict:
+    return load_folder(folder, dtype)[1]
+
+
 def rms_norm(x, weight, eps):
     """x / sqrt(mean(x^2) + eps) (* weight), over the last axis."""
     y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
@@ -71,25 +88,31 @@ def visible(n, size, keep_first):
     return (j <= i) & ((i - j < size) | (j < keep_first))
 
 
-def attention_keys_values(h, w, prefix, m, positions):
+def _rot(m):
+    rot = m.get("rot") or {}
+    return rot.get("dims", 0), rot.get("base", 10000.0)
+
+
+def attention_keys_values(h, w, prefix, m, positions, r=same):
     """The turned keys [T, G, 2, dim] and the values [T, G, vdim] a layer stores."""
     T = h.shape[0]
     G, dim, vdim = m["kv_heads"], m["dim"], m["vdim"]
     k = (h @ w[prefix + "k"].T).view(T, G * 2, dim)
-    k = turn(k, positions, m["rot"]["dims"], m["rot"]["base"]).view(T, G, 2, dim)
-    v = (h @ w[prefix + "v"].T).view(T, G, vdim)
+    k = r(turn(k, positions, *_rot(m))).view(T, G, 2, dim)
+    v = r(h @ w[prefix + "v"].T).view(T, G, vdim)
     return k, v
 
 
-def differential_attention(h, w, prefix, m, eps, positions, kv=None):
+def differential_attention(h, w, prefix, m, eps, positions, kv=None, r=same):
     """h [T, width] -> [T, width].  `kv`: another layer's (keys, values) to read in place of
     this layer's own."""
     T = h.shape[0]
     H, G, dim, vdim = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = (h @ w[prefix + "q"].T).view(T, H * 2, dim)
-    q = turn(q, positions, m["rot"]["dims"], m["rot"]["base"]).view(T, H, 2, dim)
-    k, v = kv if kv is not None else attention_keys_values(h, w, prefix, m, positions)
-    mask = visible(T, m["mask"]["size"], m["mask"]["keep_first"])
+    q = r(turn(q, positions, *_rot(m))).view(T, H, 2, dim)
+    k, v = kv if kv is not None else attention_keys_values(h, w, prefix, m, positions, r)
+    mask_cfg = m.get("mask") or {}
+    mask = visible(T, mask_cfg.get("size") or T + 1, mask_cfg.get("keep_first") or 0)
     lam = (torch.exp((w[prefix + "lq1"] * w[prefix + "lk1"]).sum())
            - torch.exp((w[prefix + "lq2"] * w[prefix + "lk2"]).sum()) + m["diff"])
     gate = torch.sigmoid(h @ w[prefix + "g"].T)                      # [T, H]
@@ -101,36 +124,40 @@ def differential_attention(h, w, prefix, m, eps, positions, kv=None):
         for which in range(2):
             score = (q[:, head, which] @ k[:, g, which].T) * m["scale"]
             score = score.masked_fill(~mask, float("-inf"))
-            maps.append(torch.softmax(score, dim=-1) @ v[:, g])
+            maps.append(r(torch.softmax(score, dim=-1) @ v[:, g]))
         o = maps[0] - lam * maps[1]
         o = rms_norm(o, None, eps) * (1.0 - m["diff"])
         out[:, head] = o * gate[:, head:head + 1]
-    return out.reshape(T, H * vdim) @ w[prefix + "o"].T
+    return r(out.reshape(T, H * vdim)) @ w[prefix + "o"].T
 
 
-def retention(h, w, prefix, m, eps, positions):
+def retention(h, w, prefix, m, eps, positions, r=same, state=None):
+    """`state` [H, dim, vdim] (default zeros) is where the recurrence starts; it is updated in
+    place, so that a sequence can be run in pieces."""
     T = h.shape[0]
     H, dim, vdim = m["heads"], m["dim"], m["vdim"]
-    q = turn((h @ w[prefix + "q"].T).view(T, H, dim), positions, m["rot"]["dims"], m["rot"]["base"])
-    k = turn((h @ w[prefix + "k"].T).view(T, H, dim), positions, m["rot"]["dims"], m["rot"]["base"])
+    q = turn((h @ w[prefix + "q"].T).view(T, H, dim), positions, *_rot(m))
+    k = turn((h @ w[prefix + "k"].T).view(T, H, dim), positions, *_rot(m))
     k = k * dim ** -0.5
     v = (h @ w[prefix + "v"].T).view(T, H, vdim)
     out = torch.empty(T, H, vdim, dtype=h.dtype)
     for head in range(H):
         decay = float(m["decay"][head])
-        state = torch.zeros(dim, vdim, dtype=h.dtype)
+        s = torch.zeros(dim, vdim, dtype=h.dtype) if state is None else state[head]
         for t in range(T):
-            state = decay * state + torch.outer(k[t, head], v[t, head])
-            out[t, head] = state.T @ q[t, head]
+            s = decay * s + torch.outer(k[t, head], v[t, head])
+            out[t, head] = s.T @ q[t, head]
+        if state is not None:
+            state[head] = s
     out = rms_norm(out, None, eps).reshape(T, H * vdim)
-    return (out * silu(h @ w[prefix + "g"].T)) @ w[prefix + "o"].T
+    return r(out * silu(h @ w[prefix + "g"].T)) @ w[prefix + "o"].T
 
 
-def gated(h, w, prefix, act):
-    return (act(h @ w[prefix + "gate"].T) * (h @ w[prefix + "up"].T)) @ w[prefix + "down"].T
+def gated(h, w, prefix, act, r=same):
+    return r(act(r(h @ w[prefix + "gate"].T)) * r(h @ w[prefix + "up"].T)) @ w[prefix + "down"].T
 
 
-def routed_experts(h, w, prefix, mlp):
+def routed_experts(h, w, prefix, mlp, r=same):
     experts, top = mlp["router"]["experts"], mlp["router"]["top"]
     logits = h @ w[prefix + "router"].T
     chosen, ids = torch.topk(logits, top, dim=-1)
@@ -139,21 +166,22 @@ def routed_experts(h, w, prefix, mlp):
     for t in range(h.shape[0]):
         for j in range(top):
             e = int(ids[t, j])
-            out[t] += weights[t, j] * gated(h[t:t + 1], w, f"{prefix}e{e}.", silu)[0]
+            out[t] += weights[t, j] * gated(h[t:t + 1], w, f"{prefix}e{e}.", silu, r)[0]
     if mlp.get("shared"):
         share = torch.sigmoid(h @ w[prefix + "shared.sg"].T)          # [T, 1]
-        out = out + share * gated(h, w, prefix + "shared.", silu)
+        out = out + share * gated(h, w, prefix + "shared.", silu, r)
     return out
 
 
-def feed_forward(h, w, prefix, mlp):
+def feed_forward(h, w, prefix, mlp, r=same):
     if mlp["kind"] == "dense":
-        return gated(h, w, prefix, gelu_tanh)
-    return routed_experts(h, w, prefix, mlp)
+        return gated(h, w, prefix, gelu_tanh, r)
+    return routed_experts(h, w, prefix, mlp, r)
 
 
-def forward(config, w, tokens, return_layers=False):
-    """Logits [T, vocab] of one sequence (and the stream after every layer)."""
+def forward(config, w, tokens, r=same, return_layers=False):
+    """Logits [T, vocab] of one sequence (and the stream after every layer).  `r` rounds what
+    enters and leaves the matrix products (`to_bf16`: what the format costs on this input)."""
     eps = config["norm"]["eps"]
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(tokens.numel())
@@ -161,22 +189,22 @@ def forward(config, w, tokens, return_layers=False):
     stored, after = {}, []
     for i, layer in enumerate(config["layers"]):
         p, m = f"l{i}.", layer["mixer"]
-        h = rms_norm(s, w[p + "norm1"], eps)
+        h = r(rms_norm(s, w[p + "norm1"], eps))
         if layer["type"] == "attention":
             source = m.get("kv_from")
             if source is None:
-                stored[i] = attention_keys_values(h, w, p + "mix.", m, positions)
+                stored[i] = attention_keys_values(h, w, p + "mix.", m, positions, r)
             y = differential_attention(h, w, p + "mix.", m, eps, positions,
-                                       kv=None if source is None else stored[source])
+                                       kv=None if source is None else stored[source], r=r)
         elif layer["type"] == "retention":
-            y = retention(h, w, p + "mix.", m, eps, positions)
+            y = retention(h, w, p + "mix.", m, eps, positions, r)
         else:
             raise ValueError(layer["type"])
         s = s + w[p + "ls1"] * rms_norm(y, w[p + "norm1b"], eps)
         if layer.get("mlp"):
-            h = rms_norm(s, w[p + "norm2"], eps)
-            y = feed_forward(h, w, p + "mlp.", layer["mlp"])
+            h = r(rms_norm(s, w[p + "norm2"], eps))
+            y = feed_forward(h, w, p + "mlp.", layer["mlp"], r)
             s = s + w[p + "ls2"] * rms_norm(y, w[p + "norm2b"], eps)
         after.append(s)
-    logits = rms_norm(s, w["final.norm"], eps) @ w["head"].T
+    logits = r(rms_norm(s, w["final.norm"], eps)) @ w["head"].T
     return (logits, torch.stack(after)) if return_layers else logits
