@@ -75,9 +75,10 @@ class ReplaySession:
             want = list(entry.get("want", []))
             if not tokens:
                 continue
-            # A place wanted twice is computed once and written twice.
+            # A place wanted twice is computed once and written twice; places are computed in
+            # rising order and written in the order they were asked for.
             once = sorted(set(want))
-            repeated = repeated or len(once) != len(want)
+            repeated = repeated or once != want
             base = sum(len(c.want) for c in chunks)
             picks.extend(base + once.index(w) for w in want)
             want = once

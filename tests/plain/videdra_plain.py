@@ -157,9 +157,20 @@ def gated(h, w, prefix, act, r=same):
     return r(act(r(h @ w[prefix + "gate"].T)) * r(h @ w[prefix + "up"].T)) @ w[prefix + "down"].T
 
 
-def routed_experts(h, w, prefix, mlp, r=same):
+def routing_gap(logits, top):
+    """[T]: how far the last chosen logit lies above the first one left out, relative to the
+    largest logit's size (1 where every expert is chosen)."""
+    if top >= logits.shape[-1]:
+        return torch.ones(logits.shape[0], dtype=logits.dtype)
+    ranked = logits.sort(-1, descending=True).values
+    return (ranked[:, top - 1] - ranked[:, top]) / ranked.abs().amax(-1).clamp_min(1e-30)
+
+
+def routed_experts(h, w, prefix, mlp, r=same, gaps=None):
     experts, top = mlp["router"]["experts"], mlp["router"]["top"]
     logits = h @ w[prefix + "router"].T
+    if gaps is not None:
+        gaps.append(routing_gap(logits, top))
     chosen, ids = torch.topk(logits, top, dim=-1)
     weights = torch.softmax(chosen, dim=-1)
     out = torch.zeros_like(h)
@@ -173,15 +184,16 @@ def routed_experts(h, w, prefix, mlp, r=same):
     return out
 
 
-def feed_forward(h, w, prefix, mlp, r=same):
+def feed_forward(h, w, prefix, mlp, r=same, gaps=None):
     if mlp["kind"] == "dense":
         return gated(h, w, prefix, gelu_tanh, r)
-    return routed_experts(h, w, prefix, mlp, r)
+    return routed_experts(h, w, prefix, mlp, r, gaps)
 
 
-def forward(config, w, tokens, r=same, return_layers=False):
+def forward(config, w, tokens, r=same, return_layers=False, gaps=None):
     """Logits [T, vocab] of one sequence (and the stream after every layer).  `r` rounds what
-    enters and leaves the matrix products (`to_bf16`: what the format costs on this input)."""
+    enters and leaves the matrix products (`to_bf16`: what the format costs on this input).
+    `gaps`, a list, receives every routed layer's routing gaps [T]."""
     eps = config["norm"]["eps"]
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(tokens.numel())
@@ -203,8 +215,16 @@ def forward(config, w, tokens, r=same, return_layers=False):
         s = s + w[p + "ls1"] * rms_norm(y, w[p + "norm1b"], eps)
         if layer.get("mlp"):
             h = r(rms_norm(s, w[p + "norm2"], eps))
-            y = feed_forward(h, w, p + "mlp.", layer["mlp"], r)
+            y = feed_forward(h, w, p + "mlp.", layer["mlp"], r, gaps)
             s = s + w[p + "ls2"] * rms_norm(y, w[p + "norm2b"], eps)
         after.append(s)
     logits = r(rms_norm(s, w["final.norm"], eps)) @ w["head"].T
     return (logits, torch.stack(after)) if return_layers else logits
+
+
+def greedy_generate(config, w, prompt, count):
+    """`count` tokens after `prompt`, each the largest logit of the whole sequence run anew."""
+    tokens = list(prompt)
+    for _ in range(count):
+        tokens.append(int(forward(config, w, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
