@@ -109,6 +109,12 @@ def parse_args(argv=None):
                         "sizes, beside Qwen2 at equal width, depth, heads and feed-forward size")
     p.add_argument("--larozen-only", default=None,
                    help="run one entry of the comparison only (e.g. small/larozen), for a profiler")
+    p.add_argument("--videdra", action="store_true",
+                   help="prompts and decode steps of the Videdra design (two-map attention in a "
+                        "window, retention, routed experts beside a shared one) at two sets of "
+                        "layer sizes, beside Larozen and Qwen2 at equal width, depth and heads")
+    p.add_argument("--videdra-only", default=None,
+                   help="run one entry of the comparison only (e.g. small/videdra-moe), for a profiler")
     p.add_argument("--serve-requests", type=int, default=64)
     p.add_argument("--serve-chunk", type=int, default=512)
     return p.parse_args(argv)
@@ -470,12 +476,61 @@ def larozen_configs(z: dict) -> dict:
     }
 
 
+# Layer sizes for `--videdra`: four layers (attention, retention, an attention that reads the
+# first layer's keys and values, retention); maps of 64 dims (a key row of 128) over values of
+# 128 in a window of 1,024 that keeps 4 tokens; retention heads of 64 x 128.
+VIDEDRA_SIZES = {
+    "small": dict(width=2048, heads=16, kv_heads=4, dim=128, ss_heads=64, ss_vdim=64, state=128,
+                  groups=4, ff=8192, vocab=32000, layers=4, map_dim=64, window=1024, keep=4,
+                  ret_heads=16, ret_dim=64, ret_vdim=128, experts=64, top=6, expert_ff=1408,
+                  shared_ff=2816),
+    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, ss_heads=128, ss_vdim=64, state=128,
+                  groups=8, ff=12288, vocab=32000, layers=4, map_dim=64, window=1024, keep=4,
+                  ret_heads=32, ret_dim=64, ret_vdim=128, experts=64, top=6, expert_ff=1536,
+                  shared_ff=3072),
+}
+
+
+def videdra_configs(z: dict) -> dict:
+    """name -> config.json of the four models compared at the sizes `z`."""
+    def attention(kv_from=None):
+        m = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["map_dim"], "vdim": z["dim"],
+             "scale": z["map_dim"] ** -0.5, "diff": 0.3,
+             "mask": {"size": z["window"], "keep_first": z["keep"]},
+             "rot": {"base": 10000.0, "dims": z["map_dim"]}}
+        return dict(m, kv_from=kv_from) if kv_from is not None else m
+
+    heads = z["ret_heads"]
+    retention = {"heads": heads, "dim": z["ret_dim"], "vdim": z["ret_vdim"],
+                 "decay": [1.0 - 2.0 ** (-5 - 4 * h / heads) for h in range(heads)],
+                 "rot": {"base": 1e6, "dims": z["ret_dim"]}}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "shared": {"ff": z["shared_ff"]},
+           "router": {"experts": z["experts"], "top": z["top"]}}
+
+    def layers(first, rest):
+        kinds = [("attention", attention()), ("retention", retention),
+                 ("attention", attention(0)), ("retention", retention)]
+        return [{"type": kind, "mixer": mixer, "mlp": first if i == 0 else rest}
+                for i, (kind, mixer) in enumerate(kinds)]
+
+    base = {"architecture": "Videdra", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}}
+    others = larozen_configs(z)
+    return {"videdra-dense": dict(base, layers=layers(dense, dense)),
+            "videdra-moe": dict(base, layers=layers(dense, moe)),
+            "larozen": others["larozen"], "qwen2": others["qwen2"]}
+
+
 def talolorn_main(args) -> int:
     return compare_main(args, "Talolorn", TALOLORN_SIZES, talolorn_configs, args.talolorn_only)
 
 
 def larozen_main(args) -> int:
     return compare_main(args, "Larozen", LAROZEN_SIZES, larozen_configs, args.larozen_only)
+
+
+def videdra_main(args) -> int:
+    return compare_main(args, "Videdra", VIDEDRA_SIZES, videdra_configs, args.videdra_only)
 
 
 def compare_main(args, design: str, sizes: dict, configs, only) -> int:
@@ -522,6 +577,8 @@ def main(argv=None) -> int:
         return talolorn_main(args)
     if args.larozen:
         return larozen_main(args)
+    if args.videdra:
+        return videdra_main(args)
     model_name, shape = SHAPES[args.shape]
     cfg = dict(shape)
     full_layers = cfg["num_hidden_layers"]

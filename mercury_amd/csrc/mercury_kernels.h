@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 32
+#define MK_ABI_VERSION 33
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit);
@@ -521,6 +521,22 @@ int mk_attention_out_max_parts(int M, int heads_per_slice);
 int mk_attention_out(const float* part_o, const float* part_ml, int parts, const void* w_o,
                      float* out, long long* fixed_out, int M, int N, int n_q, int n_kv, int d,
                      int heads_per_slice, int wide, hipStream_t stream);
+
+// Two-map (differential) attention with its tail, bfloat16 on the matrix cores: a head's key
+// row holds two score maps of map_dim dims side by side, query (head, map) lies a key row wide
+// in q [T, q_stride] at (head * 2 + map) * 2 map_dim with its own map's dims filled; both maps
+// are softmax attentions over the same values (dv wide) inside `window` (0: every earlier key)
+// beside the sequence's first `keep_first` keys; out [T, heads, dv] =
+// (a1 - lambda a2) / rms * out_scale * sigmoid(gate[t * gate_stride + head]) (gate float32 or
+// null).  positions [T] and cu_q [S + 1] describe the step; its longest sequence brings
+// max_q_len tokens.  mk_attention_maps_supported: whether the sizes are compiled.
+int mk_attention_maps_supported(int map_dim, int dv, int page_size);
+int mk_attention_maps(const void* q, int q_stride, void* out, const void* k_cache,
+                      const void* v_cache, const float* gate, int gate_stride,
+                      const int* positions, const int* cu_q, const int* block_table,
+                      int table_stride, int page_size, int heads, int kv_heads, int map_dim,
+                      int dv, float scale, int window, int keep_first, float lambda, float eps,
+                      float out_scale, int num_seqs, int max_q_len, hipStream_t stream);
 
 // @library core
 

@@ -130,11 +130,17 @@ int run_attention(const void* params, mk_op_context* ctx) {
       const Queries q = qkv_prepared(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, p.prep, arrays,
                                      &raw, &raw_stride);
       const AttendArgs a = attend_args(p);
-      const void* attended = attend(l, q, a, arrays, s);
       const float* gate = p.head_gate && raw ? raw + (raw_stride - p.prep.extra_cols) : nullptr;
       if (p.prep.maps == 1) throw KernelError("attention: a gate per head comes with two maps");
-      const void* heads = diff_heads(l, attended, s.num_tokens, p.qkv.n_q, a.v_dim(), gate,
-                                     raw_stride, p.diff_lambda, p.diff_eps, p.diff_scale);
+      // bfloat16 at sizes the matrix cores take: one kernel attends both maps and finishes the
+      // head; else the float32-arithmetic attention over the maps as heads, then the tail
+      const void* heads = attend_maps(l, q, a, arrays, s, gate, raw_stride, p.diff_lambda,
+                                      p.diff_eps, p.diff_scale);
+      if (!heads) {
+        const void* attended = attend(l, q, a, arrays, s);
+        heads = diff_heads(l, attended, s.num_tokens, p.qkv.n_q, a.v_dim(), gate, raw_stride,
+                           p.diff_lambda, p.diff_eps, p.diff_scale);
+      }
       project_into_stream(l, heads, s.num_tokens, p.w_o, ctx->hidden, p.qkv.n_q * a.v_dim(), p.b_o,
                           p.b_o_dtype, ctx->h, ctx->out_pending, ctx->out_pending_count);
       return;

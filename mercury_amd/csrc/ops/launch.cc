@@ -430,6 +430,26 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
                                 heads_per_slice, wide ? 1 : 0, l.stream()), "attention_out");
 }
 
+void* attend_maps(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
+                  const mk_step_view& step, const float* gate, int gate_stride, float lambda,
+                  float eps, float out_scale) {
+  const int heads = a.n_q / 2, map_dim = a.head_dim / 2;
+  if (l.dtype() != kBF16 || !kernels().has_mfma() || !a.plain_scores() || a.distance_slopes ||
+      a.n_q % 2 || a.head_dim % 2 || heads % a.n_kv ||
+      !kernels().mk_attention_maps_supported(map_dim, a.v_dim(), a.page_size)) {
+    return nullptr;
+  }
+  const int m = step.num_tokens;
+  void* out = l.alloc((size_t)m * heads * a.v_dim() * l.elem());
+  if (l.dry() || m == 0) return out;
+  check_mfma(kernels().mk_attention_maps(
+                 q.q, q.stride, out, a.k_cache, a.v_cache, gate, gate_stride, s.positions, s.cu_q,
+                 s.table, s.table_stride, a.page_size, heads, a.n_kv, map_dim, a.v_dim(), a.scale,
+                 a.window, a.window > 0 ? a.keep_first : 0, lambda, eps, out_scale, step.num_seqs,
+                 step.max_q_len, l.stream()), "attention");
+  return out;
+}
+
 void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float* gate,
                  int gate_stride, float lambda, float eps, float out_scale) {
   void* out = l.alloc((size_t)m * heads * dv * l.elem());

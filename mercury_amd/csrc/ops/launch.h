@@ -221,6 +221,13 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
                         AttendForce force = {}, int fold = -1, long long* h_fixed = nullptr);
 
 // Two maps per head combined: a [m, heads, 2, dv] -> [m, heads dv] in the compute dtype,
+// Two maps a head attended, combined, normed and gated in one matrix-core kernel (see
+// mk_attention_maps), or null where that kernel does not serve the step: another dtype than
+// bfloat16, the library not loaded, sizes it is not compiled for, a score that is not plain.
+// `a` describes the maps as heads (n_q = heads * 2, as `attend` takes it).
+void* attend_maps(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
+                  const mk_step_view& step, const float* gate, int gate_stride, float lambda,
+                  float eps, float out_scale);
 // (a1 - lambda a2) / rms * out_scale * sigmoid(gate) (see mk_diff_heads).
 void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float* gate,
                  int gate_stride, float lambda, float eps, float out_scale);

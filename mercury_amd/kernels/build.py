@@ -44,6 +44,7 @@ LIBRARIES = {
         "attention_mfma.hip",
         "attention_out.hip",
         "attention_latent.hip",
+        "attention_maps.hip",
         "gemm_mfma.hip",
         "gemm_batched_mfma.hip",
     ],

@@ -95,6 +95,8 @@ ATTENTION_SIZES = {
     "keeps-more-than-the-window": (64, 2, 1, 16, 40, 0.25, 0.3, (4, 11), (800.0, 4)),
     "sized": (128, 8, 2, 64, 128, 0.125, 0.3, (20, 4), (10000.0, 64)),
     "window-of-one": (64, 4, 4, 32, 8, 0.2, 0.2, (1, 1), (10000.0, 32)),
+    "maps-of-32-grouped": (64, 6, 2, 32, 64, 0.2, 0.3, (14, 2), (10000.0, 16)),
+    "maps-of-128-no-window": (128, 2, 1, 128, 64, 0.1, 0.2, None, (10000.0, 128)),
 }
 
 
@@ -130,15 +132,17 @@ EDGE_MASKS = [(12, 3), (16, 1), (17, 16), (33, 2), (5, 0)]
 
 
 @pytest.mark.parametrize("dtype", BOTH)
+@pytest.mark.parametrize("widths", [(16, 24), (32, 32), (64, 128)], ids=["maps16", "maps32", "maps64"])
 @pytest.mark.parametrize("mask", EDGE_MASKS, ids=[f"window{w}-keeps{k}" for w, k in EDGE_MASKS])
-def test_the_edges_of_a_window_and_of_the_kept_tokens_show(dtype, mask):
+def test_the_edges_of_a_window_and_of_the_kept_tokens_show(dtype, mask, widths):
     """Queries so large that a map sits on one or two keys: among a few hundred (query, head,
     map) some sit on the key just inside the window, on the one just outside, on the last kept
     token, on the first one not kept.  A mask one token wider or narrower, or one that keeps
     one token more or fewer, gives the plain implementation another result, in the prompt
     (58 tokens, two portions) and in the 38 tokens decoded one by one; the kernels give the
-    mask's own."""
-    hidden, heads, kv_heads, dim, vdim = 64, 4, 2, 16, 24
+    mask's own.  Maps of 32 and of 64 dims run on the matrix cores in bfloat16 (blocks of 32
+    keys, four wavefronts taking them in turn), maps of 16 in float32 arithmetic."""
+    hidden, heads, kv_heads, (dim, vdim) = 64, 4, 2, widths
     part = two_map_attention(hidden, heads, kv_heads, dim, vdim, 0.25, 0.3, mask, (10000.0, 8))
     params = bind_random(part, dtype, scale=0.25, seed=11)
     sharpen(part, params, dtype, ["q.weight"], 12.0)
@@ -165,11 +169,12 @@ def test_the_edges_of_a_window_and_of_the_kept_tokens_show(dtype, mask):
 
 
 @pytest.mark.parametrize("dtype", BOTH)
-def test_keys_far_back_and_at_page_borders(dtype):
+@pytest.mark.parametrize("widths", [(16, 24), (32, 64)], ids=["maps16", "maps32"])
+def test_keys_far_back_and_at_page_borders(dtype, widths):
     """No window, 330 tokens, queries so large that a map sits on one or two keys anywhere in
     the sequence: a prompt of 290, then decoding across two page borders.  The keys far back
     carry the result: without the first 200 it is another."""
-    hidden, heads, kv_heads, dim, vdim = 64, 4, 1, 16, 24
+    hidden, heads, kv_heads, (dim, vdim) = 64, 4, 1, widths
     part = two_map_attention(hidden, heads, kv_heads, dim, vdim, 0.25, 0.3, None, (10000.0, 16))
     params = bind_random(part, dtype, scale=0.25, seed=21)
     sharpen(part, params, dtype, ["q.weight"], 12.0)
