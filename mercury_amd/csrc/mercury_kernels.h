@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 33
+#define MK_ABI_VERSION 34
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit);
@@ -289,12 +289,17 @@ long long mk_ssm_state_floats(int heads, int P, int N);
 // token's position (dim j with j + rot / 2), and k is multiplied by k_scale after the turn.
 // The state of a sequence is its slot's row of `state` ([heads, dim, vdim], rows slot_stride
 // floats apart), read at the step's start and left for the next; out [T, heads vdim] float32.
+// total_chunks > 0: every sequence runs as ceil(tokens / mk_retention_chunk_tokens()) chunks
+// side by side (total_chunks of them in the step) over a workspace of
+// mk_retention_scan_workspace(...) floats; 0: token by token from the slot's state.
+int mk_retention_chunk_tokens(void);
+long long mk_retention_scan_workspace(int total_chunks, int heads, int dim, int vdim);
 int mk_retention_scan(const float* proj, int proj_stride, int q_col, int k_col, int v_col,
                       const float* decay, float k_scale, const float* cos_table,
                       const float* sin_table, int table_positions, int rot, const int* positions,
                       const int* cu_q, const int* slots, float* state, long long slot_stride,
                       int heads, int dim, int vdim, float* out, int tokens, int num_seqs,
-                      hipStream_t stream);
+                      int total_chunks, float* workspace, hipStream_t stream);
 // out[t, head, :] = y[t, head, :] / rms(y[t, head, :]) * silu(gate[t * gate_stride + head dv + .]):
 // a norm per head without a weight, then a gate (float32 columns of a projection).
 int mk_head_norm_gate(const float* y, void* out, int dtype, const float* gate, int gate_stride,

@@ -477,6 +477,21 @@ void retention(Launch& l, const void* x, int m, int hidden, const RetentionArgs&
                                            kF32, false);
   float* y = (float*)l.alloc((size_t)m * inner * 4);
   void* normed = l.alloc((size_t)m * inner * l.elem());
+  // a step with a sequence longer than a chunk runs the recurrence in chunks side by side
+  const KernelTable& core = need_core();
+  const int chunk = core.mk_retention_chunk_tokens();
+  int total_chunks = 0, longest = 0;
+  for (int i = 0; i < step.num_seqs; ++i) {
+    total_chunks += (step.counts[i] + chunk - 1) / chunk;
+    longest = std::max(longest, step.counts[i]);
+  }
+  if (longest <= chunk) total_chunks = 0;
+  float* scan_ws = nullptr;
+  if (total_chunks) {
+    const long long floats = core.mk_retention_scan_workspace(total_chunks, a.heads, a.dim, a.vdim);
+    if (floats < 0) throw KernelError("retention: the recurrence does not run these sizes");
+    scan_ws = (float*)l.alloc((size_t)floats * 4);
+  }
   if (!l.dry() && m > 0) {
     const KernelTable& t = need_core();
     if (!a.state) throw KernelError("retention: no state tensor");
@@ -484,7 +499,7 @@ void retention(Launch& l, const void* x, int m, int hidden, const RetentionArgs&
                                    a.pos.sin, a.pos.table_positions, a.pos.rotary_dim,
                                    step.positions, step.cu_q, step.state_slots, a.state,
                                    a.slot_floats, a.heads, a.dim, a.vdim, y, m, step.num_seqs,
-                                   l.stream()), "retention_scan");
+                                   total_chunks, scan_ws, l.stream()), "retention_scan");
     check_core(t.mk_head_norm_gate(y, normed, l.dtype(), proj + 2 * qk + inner, width, a.eps, m,
                                    a.heads, a.vdim, l.stream()), "head_norm_gate");
   }

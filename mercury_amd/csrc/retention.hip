@@ -13,43 +13,80 @@
 // staged in LDS, turned and scaled by the threads that stage them.  A sequence's tokens run in
 // order, so the order of every sum depends on the sizes alone: a state is the same however
 // the sequence was cut into steps and whatever else the step holds.
+//
+// A step with a sequence longer than RT_CHUNK tokens runs in chunks side by side, the decay
+// being a constant: every chunk's recurrence from a zero state (pass 1, its last state into the
+// workspace), the chunks' start states one after the other (the carry:
+// S_start(c + 1) = decay^len(c) S_start(c) + S_local(c), the last into the slot), and
+// decay^(n + 1) S_start^T q_t added to the n-th token of every chunk (pass 2).
 #include "common.h"
 #include "mercury_kernels.h"
 
 #define RT_TOKENS 16       // tokens staged at a time
 #define RT_COLUMNS 32      // columns of a head per workgroup
 #define RT_MAX_DIM 256
+#define RT_CHUNK 128       // tokens of a chunk when a step runs in chunks
 
 namespace {
 
-template <int R>
+// The sequence and the tokens of chunk `c` of the step.
+__device__ __forceinline__ void chunk_span(const int* __restrict__ cu_q, int num_seqs, int c,
+                                           int& seq, int& t_begin, int& t_end) {
+  int first = 0;
+  for (seq = 0; seq < num_seqs; ++seq) {
+    const int n = (cu_q[seq + 1] - cu_q[seq] + RT_CHUNK - 1) / RT_CHUNK;
+    if (c < first + n) break;
+    first += n;
+  }
+  if (seq >= num_seqs) {
+    t_begin = t_end = 0;
+    return;
+  }
+  t_begin = cu_q[seq] + (c - first) * RT_CHUNK;
+  t_end = min(cu_q[seq + 1], t_begin + RT_CHUNK);
+}
+
+// MODE 0: a sequence's tokens from its slot's state, which is left for the next step.
+// MODE 1: a chunk's tokens from a zero state; the chunk's last state goes to `chunks`.
+// MODE 2: a chunk's start state (from `chunks`) read by its queries: out += decay^(n + 1) S^T q.
+template <int R, int MODE>
 __global__ __launch_bounds__(256) void retention_scan_kernel(
     const float* __restrict__ proj, int proj_stride, int q_col, int k_col, int v_col,
     const float* __restrict__ decay, float k_scale, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rot, const int* __restrict__ positions,
     const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ state,
-    long long slot_stride, int heads, int dim, int vdim, float* __restrict__ out) {
+    long long slot_stride, int heads, int dim, int vdim, float* __restrict__ out,
+    float* __restrict__ chunks, int num_seqs) {
   constexpr int DIM = R * 8;     // rows the lanes of a column hold between them (>= dim)
   __shared__ __align__(16) float q_s[RT_TOKENS][DIM];
   __shared__ __align__(16) float k_s[RT_TOKENS][DIM];
   __shared__ float v_s[RT_TOKENS][RT_COLUMNS];
-  const int seq = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * RT_COLUMNS;
+  const int head = blockIdx.y, col0 = blockIdx.z * RT_COLUMNS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int local = wave * 8 + (lane & 7), col = col0 + local;
   const int slice = lane >> 3, row0 = slice * R;
-  const int t_begin = cu_q[seq], t_end = cu_q[seq + 1];
+  int seq = blockIdx.x, t_begin, t_end;
+  if (MODE == 0) {
+    t_begin = cu_q[seq];
+    t_end = cu_q[seq + 1];
+  } else {
+    chunk_span(cu_q, num_seqs, blockIdx.x, seq, t_begin, t_end);
+  }
   if (t_begin >= t_end) return;
   const float g = decay[head];
   const int half = rot / 2;
   const bool live = col < vdim;
-  float* mine = state + (size_t)slots[seq] * slot_stride + (size_t)head * dim * vdim;
+  float* mine = MODE == 0
+      ? state + (size_t)slots[seq] * slot_stride + (size_t)head * dim * vdim
+      : chunks + ((size_t)blockIdx.x * heads + head) * dim * vdim;
 
   float s[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int row = row0 + i;
-    s[i] = live && row < dim ? mine[(size_t)row * vdim + col] : 0.f;
+    s[i] = MODE != 1 && live && row < dim ? mine[(size_t)row * vdim + col] : 0.f;
   }
+  float reach = g;     // MODE 2: decay^(n + 1) at the chunk's n-th token
 
   for (int t0 = t_begin; t0 < t_end; t0 += RT_TOKENS) {
     const int count = min(RT_TOKENS, t_end - t0);
@@ -82,23 +119,25 @@ __global__ __launch_bounds__(256) void retention_scan_kernel(
       q_s[tt][row] = qv;
       k_s[tt][row] = kv;
     }
-    for (int e = tid; e < count * RT_COLUMNS; e += 256) {
+    for (int e = tid; MODE != 2 && e < count * RT_COLUMNS; e += 256) {
       const int tt = e / RT_COLUMNS, c = e - tt * RT_COLUMNS;
       v_s[tt][c] = col0 + c < vdim
           ? proj[(size_t)(t0 + tt) * proj_stride + v_col + head * vdim + col0 + c] : 0.f;
     }
     __syncthreads();
     for (int tt = 0; tt < count; ++tt) {
-      const float v = v_s[tt][local];
+      const float v = MODE != 2 ? v_s[tt][local] : 0.f;
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < R; i += 4) {
-        const float4 k4 = *(const float4*)&k_s[tt][row0 + i];
         const float4 q4 = *(const float4*)&q_s[tt][row0 + i];
-        s[i] = fmaf(k4.x, v, g * s[i]);
-        s[i + 1] = fmaf(k4.y, v, g * s[i + 1]);
-        s[i + 2] = fmaf(k4.z, v, g * s[i + 2]);
-        s[i + 3] = fmaf(k4.w, v, g * s[i + 3]);
+        if (MODE != 2) {
+          const float4 k4 = *(const float4*)&k_s[tt][row0 + i];
+          s[i] = fmaf(k4.x, v, g * s[i]);
+          s[i + 1] = fmaf(k4.y, v, g * s[i + 1]);
+          s[i + 2] = fmaf(k4.z, v, g * s[i + 2]);
+          s[i + 3] = fmaf(k4.w, v, g * s[i + 3]);
+        }
         o = fmaf(s[i], q4.x, o);
         o = fmaf(s[i + 1], q4.y, o);
         o = fmaf(s[i + 2], q4.z, o);
@@ -107,14 +146,48 @@ __global__ __launch_bounds__(256) void retention_scan_kernel(
       o += __shfl_xor(o, 8, MK_WAVE);
       o += __shfl_xor(o, 16, MK_WAVE);
       o += __shfl_xor(o, 32, MK_WAVE);
-      if (slice == 0 && live) out[(size_t)(t0 + tt) * heads * vdim + head * vdim + col] = o;
+      float* at = out + (size_t)(t0 + tt) * heads * vdim + head * vdim + col;
+      if (slice == 0 && live) {
+        if (MODE == 2) *at = fmaf(reach, o, *at);
+        else *at = o;
+      }
+      reach *= g;
     }
   }
+  if (MODE == 2) return;
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int row = row0 + i;
     if (live && row < dim) mine[(size_t)row * vdim + col] = s[i];
   }
+}
+
+// The chunks' start states, one sequence's after the other: a thread owns one entry of a
+// head's state, takes it from the slot, leaves in every chunk's place what the chunk starts
+// from, and puts what the last chunk ends with back into the slot.
+__global__ __launch_bounds__(256) void retention_carry_kernel(
+    const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ state,
+    long long slot_stride, const float* __restrict__ decay, float* __restrict__ chunks, int heads,
+    int entries) {
+  const int seq = blockIdx.x, head = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= entries) return;
+  int first = 0;
+  for (int i = 0; i < seq; ++i) first += (cu_q[i + 1] - cu_q[i] + RT_CHUNK - 1) / RT_CHUNK;
+  const int tokens = cu_q[seq + 1] - cu_q[seq];
+  if (tokens <= 0) return;
+  const float g = decay[head];
+  float* mine = state + (size_t)slots[seq] * slot_stride + (size_t)head * entries + e;
+  float s = *mine;
+  for (int done = 0, c = first; done < tokens; done += RT_CHUNK, ++c) {
+    float* at = chunks + ((size_t)c * heads + head) * entries + e;
+    const float ended = *at;
+    *at = s;
+    const int len = min(RT_CHUNK, tokens - done);
+    float reach = 1.f;
+    for (int i = 0; i < len; ++i) reach *= g;
+    s = fmaf(reach, s, ended);
+  }
+  *mine = s;
 }
 
 // One wavefront per (token, head).
@@ -145,7 +218,8 @@ extern "C" int mk_retention_scan(const float* proj, int proj_stride, int q_col, 
                                  int table_positions, int rot, const int* positions,
                                  const int* cu_q, const int* slots, float* state,
                                  long long slot_stride, int heads, int dim, int vdim, float* out,
-                                 int tokens, int num_seqs, hipStream_t stream) {
+                                 int tokens, int num_seqs, int total_chunks, float* workspace,
+                                 hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && num_seqs >= 0 && heads > 0 && dim > 0 && vdim > 0,
              "retention: bad sizes");
   MK_REQUIRE(dim <= RT_MAX_DIM, "retention: heads of %d dims exceed the supported %d", dim,
@@ -164,19 +238,44 @@ extern "C" int mk_retention_scan(const float* proj, int proj_stride, int q_col, 
              "retention: too many heads or columns");
   if (tokens == 0 || num_seqs == 0) return 0;
   MK_REQUIRE(proj && decay && cu_q && slots && state && out, "retention: null operand");
-  const dim3 grid(num_seqs, heads, (vdim + RT_COLUMNS - 1) / RT_COLUMNS);
+  MK_REQUIRE(total_chunks >= 0 && (total_chunks == 0 || workspace),
+             "retention: chunks without a workspace");
+  const int columns = (vdim + RT_COLUMNS - 1) / RT_COLUMNS;
   const int per_lane = (dim + 7) / 8;
-#define RT_LAUNCH(R)                                                                            \
-  retention_scan_kernel<R><<<grid, 256, 0, stream>>>(                                          \
+#define RT_LAUNCH_R(R, MODE, first)                                                             \
+  retention_scan_kernel<R, MODE><<<dim3(first, heads, columns), 256, 0, stream>>>(              \
       proj, proj_stride, q_col, k_col, v_col, decay, k_scale, cos_table, sin_table, rot,        \
-      positions, cu_q, slots, state, slot_stride, heads, dim, vdim, out)
-  if (per_lane <= 4) RT_LAUNCH(4);
-  else if (per_lane <= 8) RT_LAUNCH(8);
-  else if (per_lane <= 16) RT_LAUNCH(16);
-  else RT_LAUNCH(32);
+      positions, cu_q, slots, state, slot_stride, heads, dim, vdim, out, workspace, num_seqs)
+#define RT_LAUNCH(MODE, first)                                                                  \
+  do {                                                                                          \
+    if (per_lane <= 4) RT_LAUNCH_R(4, MODE, first);                                             \
+    else if (per_lane <= 8) RT_LAUNCH_R(8, MODE, first);                                        \
+    else if (per_lane <= 16) RT_LAUNCH_R(16, MODE, first);                                      \
+    else RT_LAUNCH_R(32, MODE, first);                                                          \
+  } while (0)
+  if (total_chunks == 0) {
+    RT_LAUNCH(0, num_seqs);
+    MK_LAUNCH_CHECK("retention_scan");
+    return 0;
+  }
+  RT_LAUNCH(1, total_chunks);
+  MK_LAUNCH_CHECK("retention_scan (chunks)");
+  const int entries = dim * vdim;
+  retention_carry_kernel<<<dim3(num_seqs, heads, (entries + 255) / 256), 256, 0, stream>>>(
+      cu_q, slots, state, slot_stride, decay, workspace, heads, entries);
+  MK_LAUNCH_CHECK("retention_carry");
+  RT_LAUNCH(2, total_chunks);
 #undef RT_LAUNCH
-  MK_LAUNCH_CHECK("retention_scan");
+#undef RT_LAUNCH_R
+  MK_LAUNCH_CHECK("retention_scan (start states)");
   return 0;
+}
+
+extern "C" int mk_retention_chunk_tokens(void) { return RT_CHUNK; }
+
+extern "C" long long mk_retention_scan_workspace(int total_chunks, int heads, int dim, int vdim) {
+  if (total_chunks < 0 || heads <= 0 || dim <= 0 || vdim <= 0) return -1;
+  return (long long)total_chunks * heads * dim * vdim;
 }
 
 extern "C" int mk_head_norm_gate(const float* y, void* out, int dtype, const float* gate,
