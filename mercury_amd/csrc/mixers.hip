@@ -193,6 +193,56 @@ __global__ __launch_bounds__(256) void norm_scale_add_kernel(
   }
 }
 
+// The same for rows of at most 256 NV entries, one workgroup per token: a thread keeps its
+// entries in registers between the sum of squares and the output, and the partial sums of an
+// entry are read side by side (in the same order of addition).
+#define NSA_NV 16
+template <typename TW>
+__global__ __launch_bounds__(256) void norm_scale_add_held_kernel(
+    float* __restrict__ h, const float* __restrict__ y, const float* __restrict__ partials,
+    int count, size_t stride, const void* __restrict__ weight, const float* __restrict__ scale,
+    float eps, int hidden) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * hidden;
+  float vals[NSA_NV];
+#pragma unroll
+  for (int j = 0; j < NSA_NV; ++j) {
+    const int i = threadIdx.x + j * 256;
+    vals[j] = y && i < hidden ? y[base + i] : 0.f;
+  }
+  // four partial sums of every entry are asked for at a time and added in their order
+  for (int k0 = 0; k0 < count; k0 += 4) {
+    float got[4][NSA_NV];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const float* part = partials + (size_t)min(k0 + kk, count - 1) * stride + base;
+#pragma unroll
+      for (int j = 0; j < NSA_NV; ++j) {
+        const int i = threadIdx.x + j * 256;
+        got[kk][j] = i < hidden ? part[i] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+      if (k0 + kk < count) {
+#pragma unroll
+        for (int j = 0; j < NSA_NV; ++j) vals[j] += got[kk][j];
+      }
+  }
+  float sq = 0.f;
+#pragma unroll
+  for (int j = 0; j < NSA_NV; ++j) sq += vals[j] * vals[j];
+  const float r = rsqrtf(block_sum(sq, scratch) / (float)hidden + eps);
+#pragma unroll
+  for (int j = 0; j < NSA_NV; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < hidden) {
+      const float normed = vals[j] * r * weight_at<TW>(weight, i);
+      h[base + i] += scale ? scale[i] * normed : normed;
+    }
+  }
+}
+
 // One wavefront per (token, head).
 template <typename T>
 __global__ __launch_bounds__(64) void diff_heads_kernel(
@@ -332,6 +382,16 @@ extern "C" int mk_norm_scale_add(float* h, const float* y, const float* partials
   MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "norm_scale_add: weight dtype %d",
              weight_dtype);
   if (tokens == 0) return 0;
+  if (hidden <= 256 * NSA_NV) {
+    if (weight_dtype == MK_F32)
+      norm_scale_add_held_kernel<float><<<tokens, 256, 0, stream>>>(
+          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden);
+    else
+      norm_scale_add_held_kernel<bf16_t><<<tokens, 256, 0, stream>>>(
+          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden);
+    MK_LAUNCH_CHECK("norm_scale_add");
+    return 0;
+  }
   const dim3 grid(tokens, std::max(1, std::min((hidden + 255) / 256, 512 / tokens)));
   if (weight_dtype == MK_F32)
     norm_scale_add_kernel<float><<<grid, 256, 0, stream>>>(h, y, partials, count, (size_t)stride,

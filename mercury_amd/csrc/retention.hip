@@ -176,16 +176,30 @@ __global__ __launch_bounds__(256) void retention_carry_kernel(
   const int tokens = cu_q[seq + 1] - cu_q[seq];
   if (tokens <= 0) return;
   const float g = decay[head];
+  float whole = 1.f;     // the decay over a whole chunk
+  for (int i = 0; i < RT_CHUNK; ++i) whole *= g;
   float* mine = state + (size_t)slots[seq] * slot_stride + (size_t)head * entries + e;
+  float* at = chunks + ((size_t)first * heads + head) * entries + e;
+  const size_t step = (size_t)heads * entries;
+  const int count = (tokens + RT_CHUNK - 1) / RT_CHUNK;
   float s = *mine;
-  for (int done = 0, c = first; done < tokens; done += RT_CHUNK, ++c) {
-    float* at = chunks + ((size_t)c * heads + head) * entries + e;
-    const float ended = *at;
-    *at = s;
-    const int len = min(RT_CHUNK, tokens - done);
-    float reach = 1.f;
-    for (int i = 0; i < len; ++i) reach *= g;
-    s = fmaf(reach, s, ended);
+  // eight chunks' ends are asked for at a time, so that their ways to memory overlap
+  for (int c0 = 0; c0 < count; c0 += 8) {
+    float ended[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ended[j] = c0 + j < count ? at[(size_t)(c0 + j) * step] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (c0 + j >= count) break;
+      at[(size_t)(c0 + j) * step] = s;
+      float reach = whole;
+      if (c0 + j == count - 1) {
+        const int len = tokens - (count - 1) * RT_CHUNK;
+        reach = 1.f;
+        for (int i = 0; i < len; ++i) reach *= g;
+      }
+      s = fmaf(reach, s, ended[j]);
+    }
   }
   *mine = s;
 }
