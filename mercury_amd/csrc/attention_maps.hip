@@ -43,9 +43,43 @@ struct MapsParams {
   int q_stride, gate_stride, table_stride, page_shift;
   int heads, kv_heads, window, keep_first;
   float scale_log2, lambda, eps, out_scale;
+  int splits;             // workgroups that share a tile's key blocks (a step of single tokens)
+  float* parts;           // [seq, head, split, map, 2 + DV]: maximum, sum, unnormalised result
 };
 
 #define AM_WAVES 4
+
+// The tail for one row's lanes: o = a1 / l1 - lambda a2 / l2 over the head's DV values (this
+// lane: 4 DVT of them), o / rms(o) * out_scale * sigmoid(gate), bfloat16 out.
+template <int DVT>
+__device__ __forceinline__ void finish_head(const MapsParams& p, f32x4 (&acc)[2][DVT],
+                                            const float (&lsum)[2], int token, int head, int g4,
+                                            bool row_ok) {
+  constexpr int DV = DVT * 16;
+  const float inv1 = lsum[0] > 0.f ? 1.f / lsum[0] : 0.f;
+  const float inv2 = lsum[1] > 0.f ? p.lambda / lsum[1] : 0.f;
+  float sq = 0.f;
+#pragma unroll
+  for (int t = 0; t < DVT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float o = acc[0][t][i] * inv1 - acc[1][t][i] * inv2;
+      acc[0][t][i] = o;
+      sq = __builtin_fmaf(o, o, sq);
+    }
+  sq += __shfl_xor(sq, 16, 64);
+  sq += __shfl_xor(sq, 32, 64);
+  if (!row_ok) return;
+  float mult = rsqrtf(sq / (float)DV + p.eps) * p.out_scale;
+  if (p.gate) mult *= 1.f / (1.f + expf(-p.gate[(size_t)token * p.gate_stride + head]));
+  bf16_t* orow = p.out + ((size_t)token * p.heads + head) * DV + g4 * 4;
+#pragma unroll
+  for (int t = 0; t < DVT; ++t) {
+    const uint2 packed = make_uint2(pack_bf16x2(acc[0][t][0] * mult, acc[0][t][1] * mult),
+                                    pack_bf16x2(acc[0][t][2] * mult, acc[0][t][3] * mult));
+    *(uint2*)(orow + t * 16) = packed;
+  }
+}
 
 // DKC: 32-wide chunks of a map's dims; DVT: 16-wide tiles of the values.
 template <int DKC, int DVT>
@@ -58,7 +92,8 @@ __global__ __launch_bounds__(256) void attn_maps_kernel(MapsParams p) {
   const int r = lane & 15, g4 = lane >> 4;
   const int seq = blockIdx.y, head = blockIdx.z;
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
-  const int row0 = blockIdx.x * 16;
+  const int split = blockIdx.x % p.splits;
+  const int row0 = blockIdx.x / p.splits * 16;
   if (row0 >= q_len) return;                         // the whole workgroup
   const int rows = min(16, q_len - row0);
   const bool row_ok = r < rows;
@@ -92,7 +127,7 @@ __global__ __launch_bounds__(256) void attn_maps_kernel(MapsParams p) {
   float m[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
   const float c2 = p.scale_log2;
 
-  for (int index = wave; index < blocks; index += AM_WAVES) {
+  for (int index = split * AM_WAVES + wave; index < blocks; index += AM_WAVES * p.splits) {
     const int key0 = (index < a_end ? index : b_begin + index - a_end) << 5;
     const bf16_t* kbase[2];
     const bf16_t* vbase[2];
@@ -190,6 +225,7 @@ __global__ __launch_bounds__(256) void attn_maps_kernel(MapsParams p) {
     for (int w = 0; w < AM_WAVES - 1; ++w) m_all = fmaxf(m_all, stat_s[w][map][0][r]);
     const float m_use = m_all == -INFINITY ? 0.f : m_all;
     const float mine = __builtin_amdgcn_exp2f(m[map] - m_use);
+    m[map] = m_all;
     lsum[map] *= mine;
 #pragma unroll
     for (int t = 0; t < DVT; ++t) acc[map][t] *= mine;
@@ -204,30 +240,60 @@ __global__ __launch_bounds__(256) void attn_maps_kernel(MapsParams p) {
           acc[map][t][i] = __builtin_fmaf(acc_s[w][map][t][i][lane], theirs, acc[map][t][i]);
     }
   }
-  // the tail: o = a1 - lambda a2 over the head's DV values (this lane: 4 DVT of them)
-  const float inv1 = lsum[0] > 0.f ? 1.f / lsum[0] : 0.f;
-  const float inv2 = lsum[1] > 0.f ? p.lambda / lsum[1] : 0.f;
-  float sq = 0.f;
+  if (p.splits > 1) {
+    // a step of single tokens: row 0 alone is live; its four lanes leave this split's part
+    if (r != 0) return;
 #pragma unroll
-  for (int t = 0; t < DVT; ++t)
+    for (int map = 0; map < 2; ++map) {
+      float* part = p.parts + ((((size_t)seq * p.heads + head) * p.splits + split) * 2 + map) * (2 + DV);
+      if (g4 == 0) {
+        part[0] = m[map];
+        part[1] = lsum[map];
+      }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float o = acc[0][t][i] * inv1 - acc[1][t][i] * inv2;
-      acc[0][t][i] = o;
-      sq = __builtin_fmaf(o, o, sq);
+      for (int t = 0; t < DVT; ++t)
+        *(f32x4*)(part + 2 + t * 16 + g4 * 4) = acc[map][t];
     }
-  sq += __shfl_xor(sq, 16, 64);
-  sq += __shfl_xor(sq, 32, 64);
-  if (!row_ok) return;
-  float mult = rsqrtf(sq / (float)DV + p.eps) * p.out_scale;
-  if (p.gate) mult *= 1.f / (1.f + expf(-p.gate[(size_t)token * p.gate_stride + head]));
-  bf16_t* orow = p.out + ((size_t)token * p.heads + head) * DV + g4 * 4;
-#pragma unroll
-  for (int t = 0; t < DVT; ++t) {
-    const uint2 packed = make_uint2(pack_bf16x2(acc[0][t][0] * mult, acc[0][t][1] * mult),
-                                    pack_bf16x2(acc[0][t][2] * mult, acc[0][t][3] * mult));
-    *(uint2*)(orow + t * 16) = packed;
+    return;
   }
+  finish_head<DVT>(p, acc, lsum, token, head, g4, row_ok);
+}
+
+// The splits of a step of single tokens merged in their order, and the head finished: one
+// wavefront per (sequence, head), whose lanes 0, 16, 32, 48 hold the row as in the kernel above.
+template <int DVT>
+__global__ __launch_bounds__(64) void attn_maps_merge_kernel(MapsParams p) {
+  constexpr int DV = DVT * 16;
+  const int lane = threadIdx.x, r = lane & 15, g4 = lane >> 4;
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const int token = p.cu_q[seq];
+  const bool row_ok = r == 0 && p.cu_q[seq + 1] > token;
+  f32x4 acc[2][DVT];
+  float lsum[2];
+#pragma unroll
+  for (int map = 0; map < 2; ++map) {
+    const float* base = p.parts + (((size_t)seq * p.heads + head) * p.splits * 2 + map) * (2 + DV);
+    const size_t step = (size_t)2 * (2 + DV);
+    float m_all = -INFINITY;
+    for (int s = 0; s < p.splits; ++s) m_all = fmaxf(m_all, base[s * step]);
+    const float m_use = m_all == -INFINITY ? 0.f : m_all;
+    lsum[map] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) acc[map][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < p.splits; ++s) {
+      const float* part = base + s * step;
+      const float w = __builtin_amdgcn_exp2f(part[0] - m_use);
+      lsum[map] = __builtin_fmaf(part[1], w, lsum[map]);
+#pragma unroll
+      for (int t = 0; t < DVT; ++t) {
+        const f32x4 theirs = *(const f32x4*)(part + 2 + t * 16 + g4 * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[map][t][i] = __builtin_fmaf(theirs[i], w, acc[map][t][i]);
+      }
+    }
+  }
+  // the lanes of other rows hold copies of row 0's values, which leaves the shuffles alone
+  finish_head<DVT>(p, acc, lsum, token, head, g4, row_ok);
 }
 
 #define AM_SHAPES(X) X(1, 2) X(1, 4) X(1, 8) X(2, 2) X(2, 4) X(2, 8) X(4, 4) X(4, 8)
@@ -249,7 +315,7 @@ extern "C" int mk_attention_maps(const void* q, int q_stride, void* out, const v
                                  int table_stride, int page_size, int heads, int kv_heads,
                                  int map_dim, int dv, float scale, int window, int keep_first,
                                  float lambda, float eps, float out_scale, int num_seqs,
-                                 int max_q_len, hipStream_t stream) {
+                                 int max_q_len, int splits, float* parts, hipStream_t stream) {
   MK_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
              "attention_maps: %d heads over %d kv heads", heads, kv_heads);
   MK_REQUIRE(mk_attention_maps_supported(map_dim, dv, page_size),
@@ -262,6 +328,9 @@ extern "C" int mk_attention_maps(const void* q, int q_stride, void* out, const v
              gate_stride, heads);
   MK_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && num_seqs <= 65535 && heads <= 65535,
              "attention_maps: bad step sizes");
+  MK_REQUIRE(splits >= 1 && (splits == 1 || (max_q_len == 1 && parts)),
+             "attention_maps: %d splits of the keys go with a step of single tokens and a buffer",
+             splits);
   if (num_seqs == 0 || max_q_len == 0) return 0;
   MK_REQUIRE(q && out && k_cache && v_cache && positions && cu_q && block_table,
              "attention_maps: null operand");
@@ -286,7 +355,9 @@ extern "C" int mk_attention_maps(const void* q, int q_stride, void* out, const v
   p.lambda = lambda;
   p.eps = eps;
   p.out_scale = out_scale;
-  const dim3 grid((max_q_len + 15) / 16, num_seqs, heads);
+  p.splits = splits;
+  p.parts = parts;
+  const dim3 grid((max_q_len + 15) / 16 * splits, num_seqs, heads);
 #define AM_LAUNCH(DKC, DVT)                                                    \
   if (map_dim == DKC * 32 && dv == DVT * 16) {                                 \
     attn_maps_kernel<DKC, DVT><<<grid, 64 * AM_WAVES, 0, stream>>>(p);         \
@@ -294,5 +365,19 @@ extern "C" int mk_attention_maps(const void* q, int q_stride, void* out, const v
   AM_SHAPES(AM_LAUNCH) {}
 #undef AM_LAUNCH
   MK_LAUNCH_CHECK("attention_maps");
+  if (splits > 1) {
+    const dim3 merge(num_seqs, heads);
+#define AM_MERGE(DVT)                                                   \
+  if (dv == DVT * 16) attn_maps_merge_kernel<DVT><<<merge, 64, 0, stream>>>(p); else
+    AM_MERGE(2) AM_MERGE(4) AM_MERGE(8) {}
+#undef AM_MERGE
+    MK_LAUNCH_CHECK("attention_maps (merge)");
+  }
   return 0;
+}
+
+// Floats of the buffer a step of single tokens needs for `splits` > 1.
+extern "C" long long mk_attention_maps_parts(int num_seqs, int heads, int dv, int splits) {
+  if (num_seqs < 0 || heads <= 0 || dv <= 0 || splits < 1) return -1;
+  return splits == 1 ? 0 : (long long)num_seqs * heads * splits * 2 * (2 + dv);
 }

@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 34
+#define MK_ABI_VERSION 35
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit);
@@ -535,13 +535,18 @@ int mk_attention_out(const float* part_o, const float* part_ml, int parts, const
 // (a1 - lambda a2) / rms * out_scale * sigmoid(gate[t * gate_stride + head]) (gate float32 or
 // null).  positions [T] and cu_q [S + 1] describe the step; its longest sequence brings
 // max_q_len tokens.  mk_attention_maps_supported: whether the sizes are compiled.
+// splits > 1 (a step in which every sequence brings one token): that many workgroups share a
+// (sequence, head)'s key blocks and leave parts in `parts` (mk_attention_maps_parts floats),
+// which a second kernel merges in their order.
 int mk_attention_maps_supported(int map_dim, int dv, int page_size);
+long long mk_attention_maps_parts(int num_seqs, int heads, int dv, int splits);
 int mk_attention_maps(const void* q, int q_stride, void* out, const void* k_cache,
                       const void* v_cache, const float* gate, int gate_stride,
                       const int* positions, const int* cu_q, const int* block_table,
                       int table_stride, int page_size, int heads, int kv_heads, int map_dim,
                       int dv, float scale, int window, int keep_first, float lambda, float eps,
-                      float out_scale, int num_seqs, int max_q_len, hipStream_t stream);
+                      float out_scale, int num_seqs, int max_q_len, int splits, float* parts,
+                      hipStream_t stream);
 
 // @library core
 

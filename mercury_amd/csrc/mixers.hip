@@ -197,44 +197,45 @@ __global__ __launch_bounds__(256) void norm_scale_add_kernel(
 // entries in registers between the sum of squares and the output, and the partial sums of an
 // entry are read side by side (in the same order of addition).
 #define NSA_NV 16
-template <typename TW>
+template <typename TW, int NV>
 __global__ __launch_bounds__(256) void norm_scale_add_held_kernel(
     float* __restrict__ h, const float* __restrict__ y, const float* __restrict__ partials,
     int count, size_t stride, const void* __restrict__ weight, const float* __restrict__ scale,
     float eps, int hidden) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * hidden;
-  float vals[NSA_NV];
+  float vals[NV];
 #pragma unroll
-  for (int j = 0; j < NSA_NV; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const int i = threadIdx.x + j * 256;
     vals[j] = y && i < hidden ? y[base + i] : 0.f;
   }
-  // four partial sums of every entry are asked for at a time and added in their order
-  for (int k0 = 0; k0 < count; k0 += 4) {
-    float got[4][NSA_NV];
+  // 64 / NV partial sums of every entry are asked for at a time and added in their order
+  constexpr int KB = 64 / NV;
+  for (int k0 = 0; k0 < count; k0 += KB) {
+    float got[KB][NV];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
+    for (int kk = 0; kk < KB; ++kk) {
       const float* part = partials + (size_t)min(k0 + kk, count - 1) * stride + base;
 #pragma unroll
-      for (int j = 0; j < NSA_NV; ++j) {
+      for (int j = 0; j < NV; ++j) {
         const int i = threadIdx.x + j * 256;
         got[kk][j] = i < hidden ? part[i] : 0.f;
       }
     }
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
+    for (int kk = 0; kk < KB; ++kk)
       if (k0 + kk < count) {
 #pragma unroll
-        for (int j = 0; j < NSA_NV; ++j) vals[j] += got[kk][j];
+        for (int j = 0; j < NV; ++j) vals[j] += got[kk][j];
       }
   }
   float sq = 0.f;
 #pragma unroll
-  for (int j = 0; j < NSA_NV; ++j) sq += vals[j] * vals[j];
+  for (int j = 0; j < NV; ++j) sq += vals[j] * vals[j];
   const float r = rsqrtf(block_sum(sq, scratch) / (float)hidden + eps);
 #pragma unroll
-  for (int j = 0; j < NSA_NV; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const int i = threadIdx.x + j * 256;
     if (i < hidden) {
       const float normed = vals[j] * r * weight_at<TW>(weight, i);
@@ -383,12 +384,19 @@ extern "C" int mk_norm_scale_add(float* h, const float* y, const float* partials
              weight_dtype);
   if (tokens == 0) return 0;
   if (hidden <= 256 * NSA_NV) {
-    if (weight_dtype == MK_F32)
-      norm_scale_add_held_kernel<float><<<tokens, 256, 0, stream>>>(
-          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden);
-    else
-      norm_scale_add_held_kernel<bf16_t><<<tokens, 256, 0, stream>>>(
-          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden);
+#define NSA_LAUNCH(TW, NV)                                        \
+  norm_scale_add_held_kernel<TW, NV><<<tokens, 256, 0, stream>>>( \
+      h, y, partials, count, (size_t)stride, weight, scale, eps, hidden)
+    if (weight_dtype == MK_F32) {
+      if (hidden <= 256 * 4) NSA_LAUNCH(float, 4);
+      else if (hidden <= 256 * 8) NSA_LAUNCH(float, 8);
+      else NSA_LAUNCH(float, NSA_NV);
+    } else {
+      if (hidden <= 256 * 4) NSA_LAUNCH(bf16_t, 4);
+      else if (hidden <= 256 * 8) NSA_LAUNCH(bf16_t, 8);
+      else NSA_LAUNCH(bf16_t, NSA_NV);
+    }
+#undef NSA_LAUNCH
     MK_LAUNCH_CHECK("norm_scale_add");
     return 0;
   }

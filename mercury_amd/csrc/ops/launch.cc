@@ -441,12 +441,27 @@ void* attend_maps(Launch& l, const Queries& q, const AttendArgs& a, const StepAr
   }
   const int m = step.num_tokens;
   void* out = l.alloc((size_t)m * heads * a.v_dim() * l.elem());
+  // a step of single tokens: the key blocks of a (sequence, head) go to as many workgroups as
+  // leave each of their four wavefronts a block or two, while the chip has room for them
+  int splits = 1;
+  if (step.max_q_len == 1) {
+    const int reach = a.window > 0 ? std::min(step.max_kv_len, a.window + a.keep_first + 32)
+                                   : step.max_kv_len;
+    const int blocks = (reach + 31) / 32;
+    const int room = std::max(1, 2048 / std::max(1, step.num_seqs * heads));
+    splits = std::max(1, std::min({8, (blocks + 7) / 8, room}));
+  }
+  float* parts = nullptr;
+  if (splits > 1) {
+    parts = (float*)l.alloc((size_t)kernels().mk_attention_maps_parts(step.num_seqs, heads,
+                                                                      a.v_dim(), splits) * 4);
+  }
   if (l.dry() || m == 0) return out;
   check_mfma(kernels().mk_attention_maps(
                  q.q, q.stride, out, a.k_cache, a.v_cache, gate, gate_stride, s.positions, s.cu_q,
                  s.table, s.table_stride, a.page_size, heads, a.n_kv, map_dim, a.v_dim(), a.scale,
                  a.window, a.window > 0 ? a.keep_first : 0, lambda, eps, out_scale, step.num_seqs,
-                 step.max_q_len, l.stream()), "attention");
+                 step.max_q_len, splits, parts, l.stream()), "attention");
   return out;
 }
 

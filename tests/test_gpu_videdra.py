@@ -168,6 +168,29 @@ def test_the_edges_of_a_window_and_of_the_kept_tokens_show(dtype, mask, widths):
         assert off[:prompt].max() > 0.05 and off[prompt:].max() > 0.05, f"mask {other} looks like {mask}"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16])
+@pytest.mark.parametrize("mask", [None, (700, 40)], ids=["sees-all", "window700-keeps40"])
+def test_decoding_over_many_keys_splits_them_over_workgroups(dtype, mask):
+    """A prompt of 1,900 tokens, then 24 decoded ones: a step of single tokens deals a
+    sequence's key blocks over up to eight workgroups and merges their parts."""
+    hidden, heads, kv_heads, dim, vdim = 64, 4, 2, 32, 64
+    part = two_map_attention(hidden, heads, kv_heads, dim, vdim, 0.2, 0.3, mask, (10000.0, 32))
+    params = bind_random(part, dtype, scale=0.25, seed=23)
+    sharpen(part, params, dtype, ["q.weight"], 8.0)
+    n, prompt = 1924, 1900
+    x = rnd(n, hidden, seed=24).to(dtype)
+    portions = ((0, prompt),) + tuple((i, 1) for i in range(prompt, n))
+    got = run_mixer_in_portions(part, x, dtype, hidden, pages=128, portions=portions)
+    m = attention(heads, kv_heads, dim, vdim, 0.2, 0.3, mask, (10000.0, 32))
+    at = torch.arange(n)
+
+    def run(to, r):
+        names = {k: to(v) for k, v in plain_names(params).items()}
+        return plain.differential_attention(to(x), names, "p.", m, 1e-5, at, r=r).float()
+
+    compare(got, run, dtype)
+
+
 @pytest.mark.parametrize("dtype", BOTH)
 @pytest.mark.parametrize("widths", [(16, 24), (32, 64)], ids=["maps16", "maps32"])
 def test_keys_far_back_and_at_page_borders(dtype, widths):
