@@ -10,9 +10,10 @@
 // a wavefront 8 of them by 8 slices of the state's rows, a lane one column and R = ceil(dim / 8)
 // consecutive rows, in registers for the whole step.  The sum over rows for o_t is in-lane but
 // for three exchanges across the slices.  Queries, keys and values of 16 tokens at a time are
-// staged in LDS, turned and scaled by the threads that stage them.  A sequence's tokens run in
-// order, so the order of every sum depends on the sizes alone: a state is the same however
-// the sequence was cut into steps and whatever else the step holds.
+// staged in LDS, turned and scaled by the threads that stage them (64 at a time were slower:
+// a workgroup does not compute while it stages, and fewer workgroups fit beside it).  A
+// sequence's tokens run in order, so the order of every sum depends on the sizes alone: a
+// state is the same however the sequence was cut into steps and whatever else the step holds.
 //
 // A step with a sequence longer than RT_CHUNK tokens runs in chunks side by side, the decay
 // being a constant: every chunk's recurrence from a zero state (pass 1, its last state into the
@@ -58,9 +59,10 @@ __global__ __launch_bounds__(256) void retention_scan_kernel(
     long long slot_stride, int heads, int dim, int vdim, float* __restrict__ out,
     float* __restrict__ chunks, int num_seqs) {
   constexpr int DIM = R * 8;     // rows the lanes of a column hold between them (>= dim)
-  __shared__ __align__(16) float q_s[RT_TOKENS][DIM];
-  __shared__ __align__(16) float k_s[RT_TOKENS][DIM];
-  __shared__ float v_s[RT_TOKENS][RT_COLUMNS];
+  constexpr int TOKENS = RT_TOKENS;
+  __shared__ __align__(16) float q_s[TOKENS][DIM];
+  __shared__ __align__(16) float k_s[TOKENS][DIM];
+  __shared__ float v_s[TOKENS][RT_COLUMNS];
   const int head = blockIdx.y, col0 = blockIdx.z * RT_COLUMNS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int local = wave * 8 + (lane & 7), col = col0 + local;
@@ -88,8 +90,8 @@ __global__ __launch_bounds__(256) void retention_scan_kernel(
   }
   float reach = g;     // MODE 2: decay^(n + 1) at the chunk's n-th token
 
-  for (int t0 = t_begin; t0 < t_end; t0 += RT_TOKENS) {
-    const int count = min(RT_TOKENS, t_end - t0);
+  for (int t0 = t_begin; t0 < t_end; t0 += TOKENS) {
+    const int count = min(TOKENS, t_end - t0);
     __syncthreads();
     // stage: q and k turned (k scaled), rows past dim as zeros; v of this workgroup's columns
     for (int e = tid; e < count * DIM; e += 256) {
@@ -119,14 +121,19 @@ __global__ __launch_bounds__(256) void retention_scan_kernel(
       q_s[tt][row] = qv;
       k_s[tt][row] = kv;
     }
-    for (int e = tid; MODE != 2 && e < count * RT_COLUMNS; e += 256) {
+    // the values; in pass 2, in their place, what pass 1 left in out for these columns
+    for (int e = tid; e < count * RT_COLUMNS; e += 256) {
       const int tt = e / RT_COLUMNS, c = e - tt * RT_COLUMNS;
-      v_s[tt][c] = col0 + c < vdim
-          ? proj[(size_t)(t0 + tt) * proj_stride + v_col + head * vdim + col0 + c] : 0.f;
+      float got = 0.f;
+      if (col0 + c < vdim) {
+        got = MODE == 2 ? out[(size_t)(t0 + tt) * heads * vdim + head * vdim + col0 + c]
+                        : proj[(size_t)(t0 + tt) * proj_stride + v_col + head * vdim + col0 + c];
+      }
+      v_s[tt][c] = got;
     }
     __syncthreads();
     for (int tt = 0; tt < count; ++tt) {
-      const float v = MODE != 2 ? v_s[tt][local] : 0.f;
+      const float v = v_s[tt][local];
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < R; i += 4) {
@@ -148,8 +155,7 @@ __global__ __launch_bounds__(256) void retention_scan_kernel(
       o += __shfl_xor(o, 32, MK_WAVE);
       float* at = out + (size_t)(t0 + tt) * heads * vdim + head * vdim + col;
       if (slice == 0 && live) {
-        if (MODE == 2) *at = fmaf(reach, o, *at);
-        else *at = o;
+        *at = MODE == 2 ? fmaf(reach, o, v) : o;
       }
       reach *= g;
     }
