@@ -197,7 +197,7 @@ def test_keys_far_back_and_at_page_borders(dtype, widths):
     """No window, 330 tokens, queries so large that a map sits on one or two keys anywhere in
     the sequence: a prompt of 290, then decoding across two page borders.  The keys far back
     carry the result: without the first 200 it is another."""
-    hidden, heads, kv_heads, (dim, vdim) = 64, 4, 1, widths
+    hidden, heads, kv_heads, (dim, vdim) = 64, 6, 2, widths
     part = two_map_attention(hidden, heads, kv_heads, dim, vdim, 0.25, 0.3, None, (10000.0, 16))
     params = bind_random(part, dtype, scale=0.25, seed=21)
     sharpen(part, params, dtype, ["q.weight"], 12.0)
@@ -431,7 +431,7 @@ def test_norms_around_each_sublayer_and_the_stored_scale(dtype, ff, scaled):
 
 @pytest.mark.parametrize("dtype", BOTH)
 @pytest.mark.parametrize("sizes", [(64, 6, 2, 32, 48), (100, 5, 3, 18, 22), (128, 4, 1, 40, 0),
-                                   (64, 3, 3, 24, 8), (64, 16, 3, 64, 96)],
+                                   (64, 3, 3, 24, 8), (64, 16, 3, 48, 80)],
                          ids=["two-of-six-shared", "odd-three-of-five", "one-of-four-none-shared",
                               "all-of-three", "three-of-sixteen"])
 @pytest.mark.parametrize("rows", [7, 70])
