@@ -128,6 +128,33 @@ def test_two_map_attention_alone(dtype, sizes):
     assert (plain.differential_attention(x.float(), other, "p.", m, 1e-5, at) - want).abs().max() > 1e-2
 
 
+@pytest.mark.parametrize("dim", [32, 64, 128])
+@pytest.mark.parametrize("vdim", [32, 64, 128])
+@pytest.mark.parametrize("page", [16, 64])
+def test_every_width_the_matrix_core_attention_is_compiled_for(dim, vdim, page):
+    """Maps of 32, 64 and 128 dims over values of 32, 64 and 128 in bfloat16 (one of the nine
+    pairs runs in float32 arithmetic), pages of 16 and of 64 tokens: 75 tokens in a window of
+    40 that keeps 3, in two portions, then token by token."""
+    hidden, heads, kv_heads = 64, 4, 2
+    mask, rot = (40, 3), (10000.0, dim // 2)
+    part = two_map_attention(hidden, heads, kv_heads, dim, vdim, dim ** -0.5, 0.3, mask, rot)
+    params = bind_random(part, torch.bfloat16, scale=0.25, seed=dim + vdim)
+    sharpen(part, params, torch.bfloat16, ["q.weight"], 4.0)
+    n = 75
+    x = rnd(n, hidden, seed=31).to(torch.bfloat16)
+    portions = ((0, 37), (37, 21)) + tuple((i, 1) for i in range(58, n))
+    got = run_mixer_in_portions(part, x, torch.bfloat16, hidden, pages=8 * 64 // page, page=page,
+                                portions=portions)
+    m = attention(heads, kv_heads, dim, vdim, dim ** -0.5, 0.3, mask, rot)
+    at = torch.arange(n)
+
+    def run(to, r):
+        names = {k: to(v) for k, v in plain_names(params).items()}
+        return plain.differential_attention(to(x), names, "p.", m, 1e-5, at, r=r).float()
+
+    compare(got, run, torch.bfloat16)
+
+
 EDGE_MASKS = [(12, 3), (16, 1), (17, 16), (33, 2), (5, 0)]
 
 
