@@ -75,7 +75,8 @@ def build_videdra(cfg: VidedraConfig) -> DecoderModel:
             positions[key] = RotaryPosition(dim, base, rotary_dim=dims) if dims else NoPosition()
         return positions[key]
 
-    norm = lambda: RMSNorm(cfg.width, cfg.norm_eps)
+    # x * rstd * weight in float32, rounded once where a matrix product reads it
+    norm = lambda: RMSNorm(cfg.width, cfg.norm_eps, round_once=True)
     needs = _cache_needs(cfg)
     layers, calls = [], []
     for i, entry in enumerate(cfg.layers):
