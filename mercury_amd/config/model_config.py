@@ -742,3 +742,232 @@ class VidedraConfig:
                 "layers": [{"type": layer.kind, "mixer": layer.mixer.to_dict(),
                             "mlp": None if layer.mlp is None else layer.mlp.to_dict()}
                            for layer in self.layers]}
+
+
+def _rotation(raw: dict, where: str, width: int) -> tuple:
+    """(base, dims, scaling) of a mixer's ``rot`` entry; dims 0 when there is none.  `scaling`
+    is None or (factor, low, high, original)."""
+    rot = raw.get("rot") or {}
+    dims = int(rot.get("dims", 0))
+    base = float(rot.get("base", 10000.0))
+    if dims < 0 or dims > width or dims % 2:
+        raise ConfigError(f"{where}.rot.dims {dims} must be even and within {width}")
+    if dims and not base > 0:
+        raise ConfigError(f"{where}.rot.base must be positive")
+    s = rot.get("scaling")
+    scaling = None
+    if s:
+        at = where + ".rot.scaling"
+        scaling = tuple(float(_require_in(s, key, at)) for key in ("factor", "low", "high", "original"))
+        factor, low, high, original = scaling
+        if not (factor > 0 and high > low >= 0 and original > 0):
+            raise ConfigError(f"{at}: factor > 0, high > low >= 0 and original > 0 are required")
+    return base, dims, scaling
+
+
+def _rotation_dict(base: float, dims: int, scaling) -> dict:
+    out = {"base": base, "dims": dims}
+    if scaling:
+        out["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
+    return out
+
+
+@dataclass(frozen=True)
+class GatedAttentionConfig:
+    """``layers[i].mixer`` of a Mogilorn layer of type ``attention``: grouped-query causal
+    attention with biased projections, a norm per query and key head, interleaved rotation whose
+    frequencies may be scaled, a bounded score, values that may be mixed with the first such
+    layer's, and a sigmoid gate per output column."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0       # 0: the score is not bounded
+    v_mix: bool = False
+    rot_base: float = 10000.0
+    rot_dims: int = 0          # 0: queries and keys do not turn
+    rot_scaling: tuple | None = None
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "GatedAttentionConfig":
+        need = lambda key: _require_in(raw, key, where)
+        dim = int(need("dim"))
+        base, dims, scaling = _rotation(raw, where, dim)
+        cfg = cls(heads=int(need("heads")), kv_heads=int(raw.get("kv_heads") or need("heads")),
+                  dim=dim, vdim=int(raw.get("vdim") or dim), scale=float(need("scale")),
+                  softcap=float(raw.get("softcap") or 0.0), v_mix=bool(raw.get("v_mix", False)),
+                  rot_base=base, rot_dims=dims, rot_scaling=scaling)
+        for name in ("heads", "kv_heads", "dim", "vdim"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if cfg.heads % cfg.kv_heads:
+            raise ConfigError(f"{where}: {cfg.heads} heads are not a multiple of {cfg.kv_heads} kv_heads")
+        if cfg.softcap < 0:
+            raise ConfigError(f"{where}.softcap is not negative")
+        return cfg
+
+    def to_dict(self) -> dict:
+        out = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim,
+               "scale": self.scale, "v_mix": self.v_mix}
+        if self.softcap:
+            out["softcap"] = self.softcap
+        if self.rot_dims:
+            out["rot"] = _rotation_dict(self.rot_base, self.rot_dims, self.rot_scaling)
+        return out
+
+
+@dataclass(frozen=True)
+class MatrixMemoryConfig:
+    """``layers[i].mixer`` of a Mogilorn layer of type ``mlstm``."""
+
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float = 0.0      # 0: the gates' logits are not bounded
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "MatrixMemoryConfig":
+        need = lambda key: _require_in(raw, key, where)
+        dim = int(need("dim"))
+        cfg = cls(heads=int(need("heads")), dim=dim, vdim=int(raw.get("vdim") or dim),
+                  gate_cap=float(raw.get("gate_cap") or 0.0))
+        for name in ("heads", "dim", "vdim"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if cfg.gate_cap < 0:
+            raise ConfigError(f"{where}.gate_cap is not negative")
+        return cfg
+
+    def to_dict(self) -> dict:
+        out = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim}
+        if self.gate_cap:
+            out["gate_cap"] = self.gate_cap
+        return out
+
+
+@dataclass(frozen=True)
+class WindowedLatentConfig:
+    """``layers[i].mixer`` of a Mogilorn layer of type ``latent_attention``: attention through
+    a normed latent and one rotated key part shared by the heads, queries straight from the
+    input, a sliding window, a sink per head and a sigmoid gate per output column."""
+
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    window: int = 0            # 0: every earlier token
+    rot_base: float = 10000.0
+    rot_dims: int = 0
+    rot_scaling: tuple | None = None
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "WindowedLatentConfig":
+        need = lambda key: _require_in(raw, key, where)
+        rot_dim = int(raw.get("rot_dim") or 0)
+        base, dims, scaling = _rotation(raw, where, rot_dim)
+        if raw.get("rot") is not None and "dims" not in raw["rot"]:
+            dims = rot_dim - rot_dim % 2
+        cfg = cls(heads=int(need("heads")), dim=int(need("dim")), rot_dim=rot_dim,
+                  vdim=int(need("vdim")), kv_rank=int(need("kv_rank")), scale=float(need("scale")),
+                  window=int((raw.get("mask") or {}).get("size") or 0),
+                  rot_base=base, rot_dims=dims, rot_scaling=scaling)
+        for name in ("heads", "dim", "vdim", "kv_rank"):
+            if getattr(cfg, name) <= 0:
+                raise ConfigError(f"{where}.{name} must be positive, got {getattr(cfg, name)}")
+        if cfg.rot_dim < 0 or cfg.window < 0:
+            raise ConfigError(f"{where}: rot_dim and mask.size are not negative")
+        return cfg
+
+    def to_dict(self) -> dict:
+        out = {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim,
+               "kv_rank": self.kv_rank, "scale": self.scale}
+        if self.window:
+            out["mask"] = {"size": self.window}
+        if self.rot_dims:
+            out["rot"] = _rotation_dict(self.rot_base, self.rot_dims, self.rot_scaling)
+        return out
+
+
+@dataclass(frozen=True)
+class MogilornLayerConfig:
+    kind: str                  # "attention", "mlstm" or "latent_attention"
+    mixer: object
+    ff: int                    # 0: the layer has no feed-forward
+
+
+MOGILORN_MIXERS = {"attention": GatedAttentionConfig, "mlstm": MatrixMemoryConfig,
+                   "latent_attention": WindowedLatentConfig}
+
+
+@dataclass(frozen=True)
+class MogilornConfig:
+    """The Mogilorn decoder: a scaled embedding; layers whose sublayers read the float32 stream
+    itself and whose outputs are RMS-normed (weights stored around zero) before they enter
+    it; a mixer per layer out of a gated grouped-query attention, a matrix memory with
+    per-request state and a windowed latent attention with sinks; a tanh-gelu feed-forward or
+    none; the head is the embedding, behind a final norm."""
+
+    vocab: int
+    width: int
+    norm_eps: float
+    embedding_scale: float
+    layers: tuple
+    architecture: str = "Mogilorn"
+    eos_token_ids: tuple = ()
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "MogilornConfig":
+        entries = _require(raw, "layers")
+        if not isinstance(entries, list) or not entries:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(entries):
+            where = f"layers[{i}]"
+            kind = _require_in(entry, "type", where)
+            if kind not in MOGILORN_MIXERS:
+                raise ConfigError(f"{where}.type {kind!r} is not implemented; known: "
+                                  f"{', '.join(sorted(MOGILORN_MIXERS))}")
+            mixer = MOGILORN_MIXERS[kind].from_dict(_require_in(entry, "mixer", where), where + ".mixer")
+            mlp, ff = entry.get("mlp"), 0
+            if mlp is not None:
+                if _require_in(mlp, "kind", where + ".mlp") != "dense":
+                    raise ConfigError(f"{where}.mlp.kind {mlp['kind']!r} is not implemented; known: dense")
+                ff = int(_require_in(mlp, "ff", where + ".mlp"))
+                if ff <= 0:
+                    raise ConfigError(f"{where}.mlp.ff must be positive")
+            layers.append(MogilornLayerConfig(kind, mixer, ff))
+        cfg = cls(vocab=int(_require(raw, "vocab")), width=int(_require(raw, "width")),
+                  norm_eps=float(_require_in(_require(raw, "norm"), "eps", "norm")),
+                  embedding_scale=float((raw.get("embedding") or {}).get("scale", 1.0)),
+                  layers=tuple(layers),
+                  architecture=str(raw.get("architecture") or (raw.get("architectures") or ["Mogilorn"])[0]))
+        cfg.validate()
+        return cfg
+
+    def mixing_layers(self) -> list:
+        """Indices of the attention layers whose values are mixed, the first one first."""
+        return [i for i, layer in enumerate(self.layers)
+                if layer.kind == "attention" and layer.mixer.v_mix]
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("vocab and width must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        mixing = self.mixing_layers()
+        for i in mixing[1:]:
+            first, m = self.layers[mixing[0]].mixer, self.layers[i].mixer
+            if (m.kv_heads, m.vdim) != (first.kv_heads, first.vdim):
+                raise ConfigError(f"layers[{i}].mixer mixes its values with layer {mixing[0]}'s, "
+                                  "which has other kv_heads or vdim")
+
+    def to_dict(self) -> dict:
+        return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
+                "norm": {"eps": self.norm_eps}, "embedding": {"scale": self.embedding_scale},
+                "layers": [{"type": layer.kind, "mixer": layer.mixer.to_dict(),
+                            "mlp": {"kind": "dense", "ff": layer.ff} if layer.ff else None}
+                           for layer in self.layers]}

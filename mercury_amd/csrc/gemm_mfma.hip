@@ -856,8 +856,9 @@ extern "C" int mk_qkv_skinny_normed(const long long* h64, const void* norm_w, in
 
 // ------------------------------------------------------------------------------- tiled
 
-// (EPI_RELU2: EPI_BF16 with the square of relu applied to the float32 sum before it is rounded)
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3, EPI_QKV = 4, EPI_RELU2 = 5 };
+// (EPI_RELU2, EPI_GELU: EPI_BF16 with the square of relu, or the tanh form of gelu, applied to
+// the float32 sum before it is rounded)
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3, EPI_QKV = 4, EPI_RELU2 = 5, EPI_GELU = 6 };
 
 // a / b for 0 <= a < 2^22 and 0 < b: the float quotient is off by less than one, which one
 // step either way repairs.  A dozen instructions where the general division is forty, on
@@ -1201,7 +1202,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
           v[i] = r * r;
         }
       }
-      if (EPI == EPI_BF16 || EPI == EPI_RELU2) {
+      if (EPI == EPI_GELU) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // 0.5 g (1 + tanh(z)) = g / (1 + 2^(-2 z log2 e)), z = sqrt(2/pi) (g + 0.044715 g^3)
+          const float g = v[i];
+          const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+          v[i] = g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(z * -2.88539008177792681472f));
+        }
+      }
+      if (EPI == EPI_BF16 || EPI == EPI_RELU2 || EPI == EPI_GELU) {
         bf16_t* dst = (bf16_t*)out_ + (size_t)m * ldo + n;
         if (whole) {
           *(uint2*)dst = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
@@ -1484,11 +1494,13 @@ extern "C" int mk_linear_tiled_act(const void* x, const void* w, void* out, int 
                                    int act, int config, hipStream_t stream) {
   MK_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0,
              "tiled projection: K=%d must be a multiple of 8 (M=%d N=%d)", K, M, N);
-  MK_REQUIRE(act == MK_UNARY_RELU2, "tiled projection: unknown activation %d", act);
+  MK_REQUIRE(act == MK_UNARY_RELU2 || act == MK_UNARY_GELU_TANH,
+             "tiled projection: unknown activation %d", act);
   MK_REQUIRE((M + 63) / 64 <= 65535, "tiled projection: M=%d too large for one launch", M);
   if (config < 0) config = mk_linear_tiled_config(M, N, K, 2);
   MK_REQUIRE(config < TILED_CONFIGS, "tiled projection: no configuration %d", config);
-  launch_tiled<EPI_RELU2>(config, x, w, nullptr, MK_F32, out, M, N, K, N, 1, stream);
+  if (act == MK_UNARY_RELU2) launch_tiled<EPI_RELU2>(config, x, w, nullptr, MK_F32, out, M, N, K, N, 1, stream);
+  else launch_tiled<EPI_GELU>(config, x, w, nullptr, MK_F32, out, M, N, K, N, 1, stream);
   MK_LAUNCH_CHECK("linear_tiled_act");
   return 0;
 }

@@ -102,6 +102,12 @@ typedef struct mk_op_context {
      operation keeps and a later one reads; there (outside a dry walk) only when a kind of the
      program is flagged MK_OP_KEPT_STREAM */
   float* kept;
+  /* float32 [T, carried_width] that lives for the whole step like h, for values an operation
+     leaves to later operations of the same step (the values of an attention layer that later
+     layers blend into their own); there (outside a dry walk) when the program was told a
+     width (Program::need_carried), null otherwise */
+  float* carried;
+  int carried_width;
 } mk_op_context;
 
 /* What the shape of a step is before it is packed: enough to say which tile lists an

@@ -130,7 +130,9 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
   for (const Entry& e : entries_) keeps = keeps || (e.kind.run && (e.kind.flags & MK_OP_KEPT_STREAM));
   const size_t kept_bytes = keeps ? round((size_t)step.num_tokens * hidden_ * 4) : 0;
   const size_t kept_at = own ? 0 : h_bytes + logit_bytes;
-  const size_t persistent = kept_at + kept_bytes;
+  const size_t carried_at = kept_at + kept_bytes;
+  const size_t carried_bytes = round((size_t)step.num_tokens * carried_width_ * 4);
+  const size_t persistent = carried_at + carried_bytes;
   Arena arenas[2];
   if (dry) {
     arenas[0].reset(nullptr, 0, true);
@@ -175,6 +177,8 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
   ctx.h_fixed = dry || !fixed ? nullptr : (long long*)workspace;
   ctx.logits = dry ? nullptr : (own ? state.own_logits : (float*)(workspace + h_bytes));
   ctx.kept = dry || !keeps ? nullptr : (float*)(workspace + kept_at);
+  ctx.carried = dry || !carried_width_ ? nullptr : (float*)(workspace + carried_at);
+  ctx.carried_width = carried_width_;
   ctx.alloc = &arena_alloc;
   state.h = ctx.h;
   state.logits = nullptr;

@@ -126,6 +126,11 @@ class Program {
   // `gives_x` says whether it leaves an x for the operation behind it.
   void append_caller_step(int index, bool gives_x);
 
+  // Room for float32 [T, width] that lives for a whole step beside h (op_abi.h: `carried`); the
+  // widest request counts.
+  void need_carried(int width) { carried_width_ = width > carried_width_ ? width : carried_width_; }
+  int carried_width() const { return carried_width_; }
+
   size_t size() const { return entries_.size(); }
   // Whether a step of this many tokens runs on a residual stream in fixed point: every entry
   // an operation of a kind that can, and few enough tokens for the registry's rule.
@@ -163,6 +168,7 @@ class Program {
             RunState& state, bool dry, WorkspaceNeed* need) const;
 
   int dtype_, hidden_, vocab_;
+  int carried_width_ = 0;
   std::vector<Entry> entries_;
 };
 

@@ -111,6 +111,10 @@ void bind_program(py::module_& m) {
         p.append(kind, blob.data(), blob.size());
       }, py::arg("kind"), py::arg("params"),
            "Append an operation of a registered kind with its parameter block (copied).")
+      .def("need_carried", &Program::need_carried, py::arg("width"),
+           "Room for float32 [tokens, width] that lives for a whole step, for values one "
+           "operation leaves to later ones (the widest request counts).")
+      .def_property_readonly("carried_width", &Program::carried_width)
       .def("host", [](Program& p, int index, bool gives_x) { p.append_caller_step(index, gives_x); },
            py::arg("index"), py::arg("gives_x") = false,
            "Append a step the caller runs itself between two calls of run().")

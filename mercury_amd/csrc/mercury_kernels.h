@@ -10,14 +10,19 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 35
+#define MK_ABI_VERSION 36
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit);
 // GELU_TANH is 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u.
 enum { MK_ACT_SILU = 0, MK_ACT_SWISH_CLAMP = 1, MK_ACT_GELU_TANH = 2 };
-// Activations of one operand: the square of relu.
-enum { MK_UNARY_RELU2 = 0 };
+// Activations of one operand: the square of relu; 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+enum { MK_UNARY_RELU2 = 0, MK_UNARY_GELU_TANH = 1 };
+// Gates of one number per column on a mixer's output: z sigmoid(z), or sigmoid(z).
+enum { MK_GATE_SILU = 0, MK_GATE_SIGMOID = 1 };
+// Values mixed across layers (mk_qk_prepare): none; this layer leaves its values of the step's
+// tokens in a buffer; this layer's values become (1 - lambda) v + lambda * what was left.
+enum { MK_VMIX_NONE = 0, MK_VMIX_LEAVE = 1, MK_VMIX_BLEND = 2 };
 
 #ifdef __cplusplus
 extern "C" {
@@ -215,13 +220,28 @@ int mk_fill_zero(float* p, long long n, hipStream_t stream);
 // its own first `rot` dims; q_out is then [T, n_q maps, d], query (head, map) holding its
 // map's dims in their place and zeros elsewhere, so that its product with a whole key row is
 // the map's score.
+// head_norm != 0: the norms run over every head by itself, q_norm and k_norm being weights of d
+// entries shared by the heads.  v_mode (MK_VMIX_*): the values before they are cached are left
+// in v_carry [T, n_kv dv] (float32), or blended with what lies there,
+// (1 - v_lambda) v + v_lambda v_carry.
 int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int dtype, const void* q_norm,
                   const void* k_norm, int norm_dtype, float eps, float temp_coef, int temp_every,
                   const float* cos_table, const float* sin_table, int table_positions, int rot,
                   int interleaved, const int* positions, const int* token_seq,
                   const int* block_table, int table_stride, void* k_cache, void* v_cache,
                   int page_size, int n_q, int n_kv, int d, int dv, int values_are_keys,
-                  int write_kv, int maps, int tokens, hipStream_t stream);
+                  int write_kv, int maps, int head_norm, float* v_carry, int v_mode,
+                  float v_lambda, int tokens, hipStream_t stream);
+
+// out[t, i] = a[t, i] * sigmoid(gate[t * gate_stride + i]), i < width; a and out of `dtype`
+// (they may be the same), the gate float32 columns of a projection.
+int mk_gate_mul(const void* a, int dtype, const float* gate, int gate_stride, void* out,
+                int tokens, int width, hipStream_t stream);
+
+// The residual stream as a sublayer reads it: h[i] += its `count` partial sums
+// partials[k * stride + i], and out[i] = h[i] in `dtype`, i < n.
+int mk_stream_cast(float* h, const float* partials, int count, long long stride, void* out,
+                   int dtype, long long n, hipStream_t stream);
 
 // out[i] = act(x[i]) for an activation MK_UNARY_*; x of in_dtype (float32, or the output's),
 // the result rounded once to `dtype`.
@@ -300,10 +320,27 @@ int mk_retention_scan(const float* proj, int proj_stride, int q_col, int k_col, 
                       const int* cu_q, const int* slots, float* state, long long slot_stride,
                       int heads, int dim, int vdim, float* out, int tokens, int num_seqs,
                       int total_chunks, float* workspace, hipStream_t stream);
-// out[t, head, :] = y[t, head, :] / rms(y[t, head, :]) * silu(gate[t * gate_stride + head dv + .]):
-// a norm per head without a weight, then a gate (float32 columns of a projection).
+// out[t, head, :] = y[t, head, :] / rms(y[t, head, :]) * weight[head dv + .] *
+// gate(gate[t * gate_stride + head dv + .]): a norm per head (weight float32 [heads dv], or null
+// for none), then a gate MK_GATE_* (float32 columns of a projection).
 int mk_head_norm_gate(const float* y, void* out, int dtype, const float* gate, int gate_stride,
-                      float eps, int tokens, int heads, int dv, hipStream_t stream);
+                      float eps, int tokens, int heads, int dv, const float* weight,
+                      int gate_kind, hipStream_t stream);
+
+// A matrix memory with input and forget gates and a running maximum (the mLSTM cell), per head:
+//   m_t = max(f_t + m_(t-1), i_t),  S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,
+//   n_t likewise with k_t alone,  o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6),
+// S, n and m zero before the sequence.  q (times q_scale), k, v and the raw gates a_t, b_t are
+// columns of the float32 rows of proj ([heads dim] at q_col and k_col, [heads vdim] at v_col,
+// [heads] at i_col and f_col); i_t = cap tanh(a_t / cap), f_t = logsigmoid(cap tanh(b_t / cap))
+// (gate_cap <= 0: no bound).  A sequence's state is its slot's row of `state`
+// (mk_mlstm_state_floats(...) floats, rows slot_stride apart), read at the step's start and left
+// for the next; out [T, heads vdim] float32.
+long long mk_mlstm_state_floats(int heads, int dim, int vdim);
+int mk_mlstm_scan(const float* proj, int proj_stride, int q_col, int k_col, int v_col, int i_col,
+                  int f_col, float q_scale, float gate_cap, const int* cu_q, const int* slots,
+                  float* state, long long slot_stride, int heads, int dim, int vdim, float* out,
+                  int tokens, int num_seqs, hipStream_t stream);
 // out[t, part] = y[t, part] / rms(y[t, part]) * weight[part], the row in `parts` equal parts.
 int mk_group_rmsnorm(const float* y, void* out, int dtype, const void* weight, int weight_dtype,
                      float eps, int tokens, int width, int parts, hipStream_t stream);

@@ -2,10 +2,13 @@
 // arithmetic for both storage types:
 //
 //   mk_qk_prepare      queries and keys between projection and cache: norms over the whole
-//                      projection, a temperature that grows with the position, rotation of a
-//                      head's first dims, the queries out, keys and values into the paged
-//                      cache (the values may be the keys as projected);
-//   mk_unary_act       an activation of one operand (the square of relu);
+//                      projection or over every head, a temperature that grows with the
+//                      position, rotation of a head's first dims, the queries out, keys and
+//                      values into the paged cache (the values may be the keys as projected, or
+//                      mixed with the values an earlier layer left for the same tokens);
+//   mk_unary_act       an activation of one operand (the square of relu, the tanh form of gelu);
+//   mk_gate_mul        a sigmoid gate, column by column, on a mixer's output;
+//   mk_stream_cast     the residual stream itself as a sublayer's input;
 //   mk_normed_sum      h += mult * (rmsnorm(a) * wa + rmsnorm(b) * wb): mixers side by side;
 //   mk_norm_scale_add  h += scale .* (rmsnorm(y) * w): a sublayer's output normed before it
 //                      enters the stream, times a stored vector per channel;
@@ -27,6 +30,7 @@ __device__ __forceinline__ float weight_at(const void* w, int i) {
 
 // One workgroup per token, or several that share its outputs.  The row of qkv is
 // [q: n_q d | k: n_kv d | v: n_kv dv], the last part absent when the values are the keys.
+#define QK_MAX_NORMED_HEADS 1024
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const float* __restrict__ qkv, int row_stride, T* __restrict__ q_out,
@@ -35,8 +39,10 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     int rot, int interleaved, const int* __restrict__ positions,
     const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int page_shift, int n_q, int n_kv, int d,
-    int dv, int values_are_keys, int write_kv, int maps) {
+    int dv, int values_are_keys, int write_kv, int maps, int head_norm,
+    float* __restrict__ v_carry, int v_mode, float v_lambda) {
   __shared__ float scratch[16];
+  __shared__ float head_mult[QK_MAX_NORMED_HEADS];
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = rot / 2;
@@ -47,12 +53,24 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   const float* k_src = row + qw;
 
   float q_mult = 1.f, k_mult = 1.f;
-  if (q_norm) {
+  if (head_norm) {
+    // a norm per head: the wavefronts take the heads of q, then of k, in turn
+    const int lane = threadIdx.x & (MK_WAVE - 1);
+    const int normed = n_q + (write_kv ? n_kv : 0);
+    for (int head = threadIdx.x / MK_WAVE; head < normed; head += blockDim.x / MK_WAVE) {
+      const float* src = row + (size_t)head * d;
+      float sq = 0.f;
+      for (int i = lane; i < d; i += MK_WAVE) sq += src[i] * src[i];
+      sq = wave_sum(sq);
+      if (lane == 0) head_mult[head] = rsqrtf(sq / (float)d + eps);
+    }
+    __syncthreads();
+  } else if (q_norm) {
     float sq = 0.f;
     for (int i = threadIdx.x; i < qw; i += blockDim.x) sq += row[i] * row[i];
     q_mult = rsqrtf(block_sum(sq, scratch) / (float)qw + eps);
   }
-  if (k_norm && write_kv) {
+  if (k_norm && write_kv && !head_norm) {
     float sq = 0.f;
     for (int i = threadIdx.x; i < kw; i += blockDim.x) sq += k_src[i] * k_src[i];
     k_mult = rsqrtf(block_sum(sq, scratch) / (float)kw + eps);
@@ -63,10 +81,12 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
 
   // the value of entry i of q (of k) before it turns
   auto q_at = [&](int i) {
+    if (head_norm) return row[i] * head_mult[i / d] * q_mult * weight_at<TW>(q_norm, i % d);
     const float v = row[i] * q_mult;
     return q_norm ? v * weight_at<TW>(q_norm, i) : v;
   };
   auto k_at = [&](int i) {
+    if (head_norm) return k_src[i] * head_mult[n_q + i / d] * weight_at<TW>(k_norm, i % d);
     const float v = k_src[i] * k_mult;
     return k_norm ? v * weight_at<TW>(k_norm, i) : v;
   };
@@ -114,7 +134,11 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     } else {
       const int i = idx - qo - kw;
       const int head = i / dv, j = i - head * dv;
-      Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * dv + j) * page_size + off, v_src[i]);
+      float value = v_src[i];
+      // values mixed across layers: the first layer leaves its own, a later one blends them in
+      if (v_mode == MK_VMIX_LEAVE) v_carry[(size_t)t * vw + i] = value;
+      else if (v_mode == MK_VMIX_BLEND) value = (1.f - v_lambda) * value + v_lambda * v_carry[(size_t)t * vw + i];
+      Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * dv + j) * page_size + off, value);
     }
   }
 }
@@ -129,6 +153,8 @@ __global__ void unary_act_kernel(const TI* __restrict__ x, T* __restrict__ out, 
   if (kind == MK_UNARY_RELU2) {
     const float r = fmaxf(v, 0.f);
     y = r * r;
+  } else if (kind == MK_UNARY_GELU_TANH) {
+    y = 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
   }
   Elem<T>::store(out + i, y);
 }
@@ -281,6 +307,30 @@ __global__ void copy_f32_kernel(float* __restrict__ dst, const float* __restrict
   if (i < n) dst[i] = src[i];
 }
 
+template <typename T>
+__global__ void gate_mul_kernel(const T* __restrict__ a, const float* __restrict__ gate,
+                                int gate_stride, T* __restrict__ out, int width, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long long t = i / width;
+  const float z = gate[t * gate_stride + (i - t * width)];
+  Elem<T>::store(out + i, Elem<T>::load(a + i) / (1.f + expf(-z)));
+}
+
+// h += its partial sums, and the sum goes out in the compute dtype.
+template <typename T>
+__global__ void stream_cast_kernel(float* __restrict__ h, const float* __restrict__ partials,
+                                   int count, size_t stride, T* __restrict__ out, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float v = h[i];
+  if (count > 0) {
+    for (int k = 0; k < count; ++k) v += partials[(size_t)k * stride + i];
+    h[i] = v;
+  }
+  Elem<T>::store(out + i, v);
+}
+
 }  // namespace
 
 extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int dtype,
@@ -290,9 +340,18 @@ extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int 
                              int interleaved, const int* positions, const int* token_seq,
                              const int* block_table, int table_stride, void* k_cache,
                              void* v_cache, int page_size, int n_q, int n_kv, int d, int dv,
-                             int values_are_keys, int write_kv, int maps, int tokens,
+                             int values_are_keys, int write_kv, int maps, int head_norm,
+                             float* v_carry, int v_mode, float v_lambda, int tokens,
                              hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv >= 0 && d > 0 && dv > 0, "qk_prepare: bad sizes");
+  MK_REQUIRE(!head_norm || (q_norm && (k_norm || !write_kv) && maps == 1),
+             "qk_prepare: a norm per head needs its weights and one map a head");
+  MK_REQUIRE(!head_norm || n_q + n_kv <= QK_MAX_NORMED_HEADS,
+             "qk_prepare: %d heads to norm exceed the supported %d", n_q + n_kv, QK_MAX_NORMED_HEADS);
+  MK_REQUIRE(v_mode == MK_VMIX_NONE || v_mode == MK_VMIX_LEAVE || v_mode == MK_VMIX_BLEND,
+             "qk_prepare: unknown value mixing %d", v_mode);
+  MK_REQUIRE(v_mode == MK_VMIX_NONE || (v_carry && write_kv && !values_are_keys),
+             "qk_prepare: values mixed across layers need a buffer and a layer that writes its own");
   MK_REQUIRE(maps >= 1 && d % maps == 0, "qk_prepare: %d maps do not divide a head of %d", maps, d);
   MK_REQUIRE(rot >= 0 && rot <= d / maps && rot % 2 == 0,
              "qk_prepare: rotary width %d not in [0, %d] / even", rot, d / maps);
@@ -318,7 +377,8 @@ extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int 
   qk_prepare_kernel<T, TW><<<grid, 256, 0, stream>>>(                                          \
       qkv, row_stride, (T*)q_out, q_norm, k_norm, eps, temp_coef, temp_every, cos_table,         \
       sin_table, rot, interleaved, positions, token_seq, block_table, table_stride, (T*)k_cache, \
-      (T*)v_cache, mk_log2(page_size), n_q, n_kv, d, dv, values_are_keys, write_kv, maps)
+      (T*)v_cache, mk_log2(page_size), n_q, n_kv, d, dv, values_are_keys, write_kv, maps,         \
+      head_norm, v_carry, v_mode, v_lambda)
   if (dtype == MK_F32) {
     if (norm_dtype == MK_F32) QK_LAUNCH(float, float); else QK_LAUNCH(float, bf16_t);
   } else if (dtype == MK_BF16) {
@@ -334,7 +394,7 @@ extern "C" int mk_qk_prepare(const float* qkv, int row_stride, void* q_out, int 
 extern "C" int mk_unary_act(const void* x, int in_dtype, void* out, int dtype, long long n,
                             int kind, hipStream_t stream) {
   MK_REQUIRE(n >= 0, "unary_act: negative count");
-  MK_REQUIRE(kind == MK_UNARY_RELU2, "unary_act: unknown activation %d", kind);
+  MK_REQUIRE(kind == MK_UNARY_RELU2 || kind == MK_UNARY_GELU_TANH, "unary_act: unknown activation %d", kind);
   if (n == 0) return 0;
   const long long blocks = (n + 255) / 256;
   MK_REQUIRE(blocks < (1ll << 31), "unary_act: %lld elements are too many for one launch", n);
@@ -452,5 +512,40 @@ extern "C" int mk_copy_f32(float* dst, const float* src, long long n, hipStream_
   MK_REQUIRE(blocks < (1ll << 31), "copy: %lld elements are too many for one launch", n);
   copy_f32_kernel<<<(unsigned)blocks, 256, 0, stream>>>(dst, src, n);
   MK_LAUNCH_CHECK("copy");
+  return 0;
+}
+
+extern "C" int mk_gate_mul(const void* a, int dtype, const float* gate, int gate_stride, void* out,
+                           int tokens, int width, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && width > 0, "gate_mul: bad sizes");
+  MK_REQUIRE(gate_stride >= width, "gate_mul: gate rows of %d for %d columns", gate_stride, width);
+  if (tokens == 0) return 0;
+  MK_REQUIRE(a && gate && out, "gate_mul: null operand");
+  const long long n = (long long)tokens * width, blocks = (n + 255) / 256;
+  MK_REQUIRE(blocks < (1ll << 31), "gate_mul: %lld elements are too many for one launch", n);
+  if (dtype == MK_F32)
+    gate_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)a, gate, gate_stride, (float*)out, width, n);
+  else if (dtype == MK_BF16)
+    gate_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)a, gate, gate_stride, (bf16_t*)out, width, n);
+  else
+    MK_REQUIRE(false, "gate_mul: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("gate_mul");
+  return 0;
+}
+
+extern "C" int mk_stream_cast(float* h, const float* partials, int count, long long stride,
+                              void* out, int dtype, long long n, hipStream_t stream) {
+  MK_REQUIRE(n >= 0 && count >= 0 && (count == 0 || partials), "stream_cast: bad operands");
+  if (n == 0) return 0;
+  MK_REQUIRE(h && out, "stream_cast: null operand");
+  const long long blocks = (n + 255) / 256;
+  MK_REQUIRE(blocks < (1ll << 31), "stream_cast: %lld elements are too many for one launch", n);
+  if (dtype == MK_F32)
+    stream_cast_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(h, partials, count, (size_t)stride, (float*)out, n);
+  else if (dtype == MK_BF16)
+    stream_cast_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>(h, partials, count, (size_t)stride, (bf16_t*)out, n);
+  else
+    MK_REQUIRE(false, "stream_cast: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("stream_cast");
   return 0;
 }

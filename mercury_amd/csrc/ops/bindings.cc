@@ -247,6 +247,23 @@ void bind_ops(py::module_& m) {
     p.prep.maps = get<int>(d, "maps", 1);
     p.head_gate = get<bool>(d, "head_gate", false) ? 1 : 0;
     p.prep.extra_cols = p.head_gate ? p.qkv.n_q : 0;
+    p.out_gate = get<bool>(d, "out_gate", false) ? 1 : 0;
+    if (p.out_gate) {
+      if (p.head_gate) throw KernelError("attention: a gate per head or a gate per column, not both");
+      p.prep.extra_cols = p.qkv.n_q * (p.prep.value_dim > 0 ? p.prep.value_dim : p.qkv.head_dim);
+    }
+    p.prep.head_norm = get<bool>(d, "head_norm", false) ? 1 : 0;
+    if (p.prep.head_norm && (!p.prep.q_norm || p.prep.maps != 1)) {
+      throw KernelError("attention: a norm per head needs its weights and one map a head");
+    }
+    p.prep.v_mode = get<int>(d, "v_mode", 0);
+    p.prep.v_lambda = get<float>(d, "v_lambda", 0.f);
+    if (p.prep.v_mode < MK_VMIX_NONE || p.prep.v_mode > MK_VMIX_BLEND) {
+      throw KernelError("attention: unknown value mixing " + std::to_string(p.prep.v_mode));
+    }
+    if (p.prep.v_mode && (!p.qkv.writes || p.prep.values_are_keys)) {
+      throw KernelError("attention: values mixed across layers are a layer's own projected values");
+    }
     p.keep_first = get<int>(d, "keep_first", 0);
     p.diff_lambda = get<float>(d, "diff_lambda", 0.f);
     p.diff_eps = get<float>(d, "diff_eps", 0.f);
@@ -267,7 +284,9 @@ void bind_ops(py::module_& m) {
     return blob(p);
   });
   m.def("unary_mlp_params", [](uintptr_t w_up, uintptr_t w_down, int inter, int act) {
-    if (act != MK_UNARY_RELU2) throw KernelError("unknown activation " + std::to_string(act));
+    if (act != MK_UNARY_RELU2 && act != MK_UNARY_GELU_TANH) {
+      throw KernelError("unknown activation " + std::to_string(act));
+    }
     UnaryMlpParams p;
     p.w_up = as_ptr<const void>(w_up);
     p.w_down = as_ptr<const void>(w_down);
@@ -333,6 +352,34 @@ void bind_ops(py::module_& m) {
     }
     if (get<bool>(d, "interleaved", false)) {
       throw KernelError("retention: queries and keys turn in the half-split layout");
+    }
+    return blob(p);
+  });
+  m.def("stream_cast_params", []() { return blob(StreamCastParams()); });
+  m.def("mlstm_state_floats", [](int heads, int dim, int vdim) {
+    const long long n = need_core().mk_mlstm_state_floats(heads, dim, vdim);
+    if (n < 0) throw KernelError("mlstm: the recurrence does not run these sizes");
+    return n;
+  }, "Floats of state a request holds for `heads` heads of a [dim, vdim] memory with n and m.");
+  m.def("mlstm_params", [](const py::kwargs& kw) {
+    const py::dict d = kw;
+    MlstmParams p;
+    MlstmArgs& a = p.args;
+    a.w_in = ptr_of<const void>(d, "w_in");
+    a.b_in = ptr_of<const void>(d, "b_in");
+    a.b_in_dtype = get<int>(d, "b_in_dtype", kF32);
+    a.w_out = ptr_of<const void>(d, "w_out");
+    a.norm = ptr_of<const float>(d, "norm");
+    a.heads = get<int>(d, "heads", 0);
+    a.dim = get<int>(d, "dim", 0);
+    a.vdim = get<int>(d, "vdim", 0);
+    a.q_scale = get<float>(d, "q_scale", 1.f);
+    a.gate_cap = get<float>(d, "gate_cap", 0.f);
+    a.eps = get<float>(d, "eps", 0.f);
+    a.state = ptr_of<float>(d, "state");
+    a.slot_floats = get<long long>(d, "slot_floats", 0);
+    if (a.heads <= 0 || a.dim <= 0 || a.vdim <= 0 || !a.w_in || !a.w_out) {
+      throw KernelError("mlstm: bad sizes");
     }
     return blob(p);
   });
@@ -438,12 +485,16 @@ void bind_ops(py::module_& m) {
     a.writes = get<bool>(d, "writes", true);
     p.w_o = ptr_of<const void>(d, "w_o");
     p.group = get<int>(d, "group", 0);
-    p.window = get<int>(d, "window", 0);
+    a.window = get<int>(d, "window", 0);
+    a.sinks = ptr_of<const float>(d, "sinks");
+    p.out_gate = get<bool>(d, "out_gate", false) ? 1 : 0;
+    a.gate_cols = p.out_gate ? a.heads * a.vdim : 0;
     p.scale = get<float>(d, "scale", 0.f);
-    if (a.heads <= 0 || a.dim <= 0 || a.vdim <= 0 || a.q_rank <= 0 || a.kv_rank <= 0 || a.rot < 0 ||
-        a.pos.rotary_dim > a.rot) {
+    if (a.heads <= 0 || a.dim <= 0 || a.vdim <= 0 || a.q_rank < 0 || a.kv_rank <= 0 || a.rot < 0 ||
+        a.pos.rotary_dim > a.rot || a.window < 0) {
       throw KernelError("latent attention: bad sizes");
     }
+    if (a.q_rank > 0 && (!a.q_norm || !a.w_uq)) throw KernelError("latent attention: no query latent's norm");
     return blob(p);
   });
   m.def("routed_experts_params", [](const py::kwargs& kw) {

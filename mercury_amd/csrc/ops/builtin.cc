@@ -122,6 +122,23 @@ int run_attention(const void* params, mk_op_context* ctx) {
       throw KernelError("attention: norms over q and k, a query temperature or values that are "
                         "keys do not run on a stream in fixed point");
     }
+    if (p.out_gate) {
+      // a sigmoid gate on every column of the heads' outputs, its logits the last columns of
+      // the stacked projection
+      if (p.prep.maps != 1 || p.head_gate) throw KernelError("attention: one gate, and one map a head with it");
+      const float* raw = nullptr;
+      int raw_stride = 0;
+      const Queries q = qkv_prepared(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, p.prep, arrays,
+                                     &raw, &raw_stride);
+      const AttendArgs a = attend_args(p);
+      const int inner = p.qkv.n_q * a.v_dim();
+      const void* attended = attend(l, q, a, arrays, s);
+      const void* gated = gate_mul(l, attended, s.num_tokens, inner,
+                                   raw ? raw + (raw_stride - inner) : nullptr, raw_stride);
+      project_into_stream(l, gated, s.num_tokens, p.w_o, ctx->hidden, inner, p.b_o, p.b_o_dtype,
+                          ctx->h, ctx->out_pending, ctx->out_pending_count);
+      return;
+    }
     if (p.prep.maps > 1 || p.head_gate) {
       // maps combined, normed per head and gated between the attention and its projection
       if (p.prep.maps != 1 && p.prep.maps != 2) throw KernelError("attention: one or two maps a head");
@@ -194,10 +211,17 @@ int run_latent_attention(const void* params, mk_op_context* ctx) {
     if (ctx->x_rows != s.num_tokens) throw KernelError("attention reads an x of every token");
     Launch l(ctx);
     const StepArrays arrays = arrays_of(s, p.group);
-    const Queries q = latent_queries(l, ctx->x, s.num_tokens, ctx->hidden, a, arrays);
-    if (p.window) throw KernelError("latent attention sees every earlier token: no window");
+    const float* raw = nullptr;
+    int raw_stride = 0;
+    const Queries q = latent_queries(l, ctx->x, s.num_tokens, ctx->hidden, a, arrays, &raw, &raw_stride);
     const void* summed = latent_attend(l, q, a, p.scale, arrays, s);
     const void* values = latent_values(l, summed, s.num_tokens, a);
+    if (p.out_gate) {
+      const int inner = a.heads * a.vdim;
+      if (a.gate_cols != inner) throw KernelError("latent attention: a gate column per value column");
+      values = gate_mul(l, values, s.num_tokens, inner, raw ? raw + (raw_stride - inner) : nullptr,
+                        raw_stride);
+    }
     project_into_stream(l, values, s.num_tokens, p.w_o, ctx->hidden, a.heads * a.vdim, nullptr, kF32,
                         ctx->h, ctx->out_pending, ctx->out_pending_count);
   });
@@ -226,6 +250,27 @@ int run_routed_experts(const void* params, mk_op_context* ctx) {
     Launch l(ctx);
     routed_experts(l, ctx->x, m, ctx->hidden, p.experts, ctx->h, ctx->out_pending,
                    ctx->out_pending_count);
+  });
+}
+
+int run_stream_cast(const void*, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    Launch l(ctx);
+    const int tokens = ctx->step->num_tokens;
+    ctx->out_x = stream_cast(l, ctx->h, tokens, ctx->hidden, ctx->pending, ctx->pending_count);
+    ctx->out_x_rows = tokens;
+    ctx->out_x_live = 1;
+  });
+}
+
+int run_mlstm(const void* params, mk_op_context* ctx) {
+  return guarded(ctx, [&] {
+    const MlstmParams& p = *static_cast<const MlstmParams*>(params);
+    const mk_step_view& s = *ctx->step;
+    if (ctx->x_rows != s.num_tokens) throw KernelError("the mixer reads an x of every token");
+    Launch l(ctx);
+    mlstm(l, ctx->x, s.num_tokens, ctx->hidden, p.args, s, ctx->h, ctx->out_pending,
+          ctx->out_pending_count);
   });
 }
 
@@ -488,6 +533,8 @@ void register_builtin_ops() {
   r.add(OpKind{"state_space", &run_state_space, nullptr, MK_OP_READS_X});
   r.add(OpKind{"normed_sum", &run_normed_sum, &tiles_normed_sum, MK_OP_READS_X});
   r.add(OpKind{"retention", &run_retention, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"mlstm", &run_mlstm, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"stream_cast", &run_stream_cast, nullptr, MK_OP_FOLDS_PENDING});
   r.add(OpKind{"post_norm", &run_post_norm, &tiles_post_norm, MK_OP_READS_X});
   r.add(OpKind{"keep_stream", &run_keep_stream, nullptr, MK_OP_KEPT_STREAM | MK_OP_FOLDS_PENDING});
   r.add(OpKind{"stream_mix", &run_stream_mix, nullptr, MK_OP_KEPT_STREAM | MK_OP_FOLDS_PENDING});

@@ -44,6 +44,22 @@ struct AttentionParams {
   // head's output is multiplied by its sigmoid (with or without two maps).
   float diff_lambda = 0.f, diff_eps = 0.f, diff_scale = 1.f;
   int head_gate = 0;
+  // out_gate: the stacked projection ends in one gate column per column of the heads side by
+  // side (n_q value_dim of them), and the attention's output is multiplied by their sigmoid
+  // before the output projection.
+  int out_gate = 0;
+};
+
+// "stream_cast": x = h + pending in the compute dtype: a sublayer that reads the residual
+// stream itself, with no norm before it.
+struct StreamCastParams {
+  int unused = 0;
+};
+
+// "mlstm": a matrix memory with gates per head and request (launch.h), its output projection
+// into h (or left as partial sums).
+struct MlstmParams {
+  MlstmArgs args;
 };
 
 // "retention": a decayed outer-product state per head and request (launch.h), its output
@@ -116,8 +132,10 @@ struct LatentAttentionParams {
   LatentArgs latent;
   const void* w_o = nullptr;   // [hidden, heads vdim]
   int group = 0;               // which of the step's block tables
-  int window = 0;
   float scale = 0.f;
+  // the down-projection ends in heads vdim gate columns whose sigmoid multiplies the heads'
+  // values before the output projection
+  int out_gate = 0;
 };
 
 // "routed_experts": h += sum over a token's chosen experts (launch.h).

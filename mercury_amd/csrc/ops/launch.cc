@@ -253,6 +253,10 @@ Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, c
   if (raw_stride) *raw_stride = width;
   void* q = l.alloc((size_t)m * a.n_q * maps * d * l.elem());
   if (l.dry() || m == 0) return {q, a.n_q * maps * d};
+  if (prep.v_mode != 0 && (!l.ctx->carried || l.ctx->carried_width < heads_kv * dv)) {
+    throw KernelError("attention: values mixed across layers need room in the step for " +
+                      std::to_string(heads_kv * dv) + " floats a token");
+  }
   const PositionDesc& p = a.pos;
   check_core(need_core().mk_qk_prepare(
                  qkv, width, q, l.dtype(), prep.q_norm, prep.k_norm, prep.norm_dtype, prep.eps,
@@ -260,7 +264,8 @@ Queries qkv_prepared(Launch& l, const void* x, int m, int k, const QkvArgs& a, c
                  p.interleaved ? 1 : 0, s.positions, s.token_seq, s.table, s.table_stride,
                  a.writes ? a.k_cache : nullptr, a.writes ? a.v_cache : nullptr,
                  a.writes ? a.page_size : 1, a.n_q, heads_kv, d, dv, prep.values_are_keys,
-                 a.writes ? 1 : 0, maps, m, l.stream()), "qk_prepare");
+                 a.writes ? 1 : 0, maps, prep.head_norm, l.ctx->carried, prep.v_mode,
+                 prep.v_lambda, m, l.stream()), "qk_prepare");
   return {q, a.n_q * maps * d};
 }
 
@@ -465,6 +470,24 @@ void* attend_maps(Launch& l, const Queries& q, const AttendArgs& a, const StepAr
   return out;
 }
 
+void* gate_mul(Launch& l, const void* a, int m, int width, const float* gate, int gate_stride) {
+  void* out = l.alloc((size_t)m * width * l.elem());
+  if (l.dry() || m == 0) return out;
+  check_core(need_core().mk_gate_mul(a, l.dtype(), gate, gate_stride, out, m, width, l.stream()),
+             "gate_mul");
+  return out;
+}
+
+void* stream_cast(Launch& l, float* h, int tokens, int hidden, const float* pending,
+                  int pending_count) {
+  void* out = l.alloc((size_t)tokens * hidden * l.elem());
+  if (l.dry() || tokens == 0) return out;
+  const long long n = (long long)tokens * hidden;
+  check_core(need_core().mk_stream_cast(h, pending, pending_count, n, out, l.dtype(), n,
+                                        l.stream()), "stream_cast");
+  return out;
+}
+
 void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float* gate,
                  int gate_stride, float lambda, float eps, float out_scale) {
   void* out = l.alloc((size_t)m * heads * dv * l.elem());
@@ -516,7 +539,33 @@ void retention(Launch& l, const void* x, int m, int hidden, const RetentionArgs&
                                    a.slot_floats, a.heads, a.dim, a.vdim, y, m, step.num_seqs,
                                    total_chunks, scan_ws, l.stream()), "retention_scan");
     check_core(t.mk_head_norm_gate(y, normed, l.dtype(), proj + 2 * qk + inner, width, a.eps, m,
-                                   a.heads, a.vdim, l.stream()), "head_norm_gate");
+                                   a.heads, a.vdim, nullptr, MK_GATE_SILU, l.stream()),
+               "head_norm_gate");
+  }
+  project_into_stream(l, normed, m, a.w_out, hidden, inner, nullptr, kF32, h, pending,
+                      pending_count);
+}
+
+void mlstm(Launch& l, const void* x, int m, int hidden, const MlstmArgs& a,
+           const mk_step_view& step, float* h, const float*& pending, int& pending_count) {
+  pending = nullptr;
+  pending_count = 0;
+  const int width = a.in_width(), qk = a.heads * a.dim, inner = a.heads * a.vdim;
+  const float* proj = (const float*)linear(l, x, m, a.w_in, width, hidden, a.b_in, a.b_in_dtype,
+                                           nullptr, kF32, false);
+  float* y = (float*)l.alloc((size_t)m * inner * 4);
+  void* normed = l.alloc((size_t)m * inner * l.elem());
+  if (!l.dry() && m > 0) {
+    const KernelTable& t = need_core();
+    if (!a.state) throw KernelError("mlstm: no state tensor");
+    const int gates = 2 * qk + 2 * inner;
+    check_core(t.mk_mlstm_scan(proj, width, 0, qk, 2 * qk, gates, gates + a.heads, a.q_scale,
+                               a.gate_cap, step.cu_q, step.state_slots, a.state, a.slot_floats,
+                               a.heads, a.dim, a.vdim, y, m, step.num_seqs, l.stream()),
+               "mlstm_scan");
+    check_core(t.mk_head_norm_gate(y, normed, l.dtype(), proj + 2 * qk + inner, width, a.eps, m,
+                                   a.heads, a.vdim, a.norm, MK_GATE_SIGMOID, l.stream()),
+               "head_norm_gate");
   }
   project_into_stream(l, normed, m, a.w_out, hidden, inner, nullptr, kF32, h, pending,
                       pending_count);
@@ -669,13 +718,15 @@ void* linear_per_head(Launch& l, const void* x, int m, int heads, int lda, int x
 }
 
 Queries latent_queries(Launch& l, const void* x, int m, int hidden, const LatentArgs& a,
-                       const StepArrays& s) {
-  const int down_width = a.q_rank + (a.writes ? a.kv_rank + a.rot : 0);
+                       const StepArrays& s, const float** raw, int* raw_stride) {
+  const int down_width = a.q_rank + (a.writes ? a.kv_rank + a.rot : 0) + a.gate_cols;
   const int per_head = a.dim + a.rot, width = a.key_width();
   // the latents in float32: the norms read them
   const float* down = (const float*)linear(l, x, m, a.w_down, down_width, hidden, nullptr, kF32,
                                            nullptr, kF32, false);
-  void* q_latent = l.alloc((size_t)m * a.q_rank * l.elem());
+  if (raw) *raw = down;
+  if (raw_stride) *raw_stride = down_width;
+  void* q_latent = a.q_rank > 0 ? l.alloc((size_t)m * a.q_rank * l.elem()) : nullptr;
   if (!l.dry() && m > 0) {
     check_core(need_core().mk_latent_prepare(
                    down, down_width, a.q_rank, a.kv_rank, a.rot, a.q_norm, a.kv_norm, a.norm_dtype,
@@ -685,8 +736,10 @@ Queries latent_queries(Launch& l, const void* x, int m, int hidden, const Latent
                    a.value_width(), l.dtype(), a.writes ? a.page_size : 1, a.writes ? 1 : 0, m,
                    l.stream()), "latent_prepare");
   }
-  const void* q = linear(l, q_latent, m, a.w_uq, a.heads * per_head, a.q_rank, nullptr, kF32,
-                         nullptr, l.dtype(), false);
+  const void* q = a.q_rank > 0
+      ? linear(l, q_latent, m, a.w_uq, a.heads * per_head, a.q_rank, nullptr, kF32, nullptr,
+               l.dtype(), false)
+      : linear(l, x, m, a.w_uq, a.heads * per_head, hidden, nullptr, kF32, nullptr, l.dtype(), false);
   void* out = l.alloc((size_t)m * a.heads * width * l.elem());
   linear_per_head(l, q, m, a.heads, a.heads * per_head, per_head, a.w_uk_t, a.kv_rank, a.dim, out,
                   a.heads * width, width);
@@ -709,6 +762,8 @@ constexpr int kLatentMinBlocks = 4;
 LatentPlan latent_plan(int dtype, const LatentArgs& a, const mk_step_view& step) {
   LatentPlan plan;
   if (dtype != kBF16 || !kernels().has_mfma()) return plan;
+  // a window or sinks: the float32-arithmetic kernel
+  if (a.window > 0 || a.sinks != nullptr) return plan;
   const KernelTable& t = need_mfma();
   if (!t.mk_attention_latent_supported(a.key_width(), a.value_width(), a.page_size)) return plan;
   plan.mfma = true;
@@ -739,7 +794,7 @@ void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scal
       check_core(need_core().mk_attention_generic_kv(
                      q.q, q.stride, out, a.heads * dv, a.k_cache, a.v_cache, l.dtype(), s.positions,
                      s.token_seq, s.table, s.table_stride, a.page_size, a.heads, 1, dk, dv, scale,
-                     0, 0, 0.f, nullptr, nullptr, m, l.stream()), "latent_attention");
+                     a.window, 0, 0.f, nullptr, a.sinks, m, l.stream()), "latent_attention");
     }
     return out;
   }

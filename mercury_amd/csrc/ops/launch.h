@@ -156,9 +156,16 @@ struct QkPrep {
   // Further columns of the stacked projection behind q, k, v that belong to the caller (a
   // gate's logits): projected in the same product, left alone here.
   int extra_cols = 0;
+  // The norms run over every head by itself, q_norm and k_norm being [head_dim] weights the
+  // heads share.
+  int head_norm = 0;
+  // Values mixed across layers (MK_VMIX_*): this layer leaves its values of the step's tokens in
+  // the step's carried buffer, or caches (1 - v_lambda) v + v_lambda * what lies there.
+  int v_mode = 0;
+  float v_lambda = 0.f;
   bool active() const {
     return q_norm != nullptr || temp_every > 0 || values_are_keys != 0 || value_dim > 0 ||
-           maps > 1 || extra_cols > 0;
+           maps > 1 || extra_cols > 0 || v_mode != 0;
   }
 };
 // qkv_project for such an attention: the projection in float32, then one kernel for all of
@@ -228,6 +235,12 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
 void* attend_maps(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
                   const mk_step_view& step, const float* gate, int gate_stride, float lambda,
                   float eps, float out_scale);
+// a .* sigmoid(gate): [m, width] of the compute dtype times the sigmoid of float32 columns
+// (rows gate_stride apart), into a new tensor.
+void* gate_mul(Launch& l, const void* a, int m, int width, const float* gate, int gate_stride);
+// The residual stream itself as a sublayer's input: h += pending, x = h in the compute dtype.
+void* stream_cast(Launch& l, float* h, int tokens, int hidden, const float* pending,
+                  int pending_count);
 // (a1 - lambda a2) / rms * out_scale * sigmoid(gate) (see mk_diff_heads).
 void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float* gate,
                  int gate_stride, float lambda, float eps, float out_scale);
@@ -254,6 +267,25 @@ struct RetentionArgs {
 };
 void retention(Launch& l, const void* x, int m, int hidden, const RetentionArgs& a,
                const mk_step_view& step, float* h, const float*& pending, int& pending_count);
+
+// A matrix memory with gates (the mLSTM cell, see mk_mlstm_scan): one projection
+// [q | k | v | gate | i | f] in float32 with a bias on its last 2 heads columns, the recurrence
+// per head from the state earlier steps left, a norm per head with a weight over all heads'
+// columns, the gate sigmoid(gate columns), the output projection into h.
+struct MlstmArgs {
+  const void* w_in = nullptr;      // [2 heads dim + 2 heads vdim + 2 heads, hidden]
+  const void* b_in = nullptr;      // [the same rows], zero but for the gates' rows
+  int b_in_dtype = 0;
+  const void* w_out = nullptr;     // [hidden, heads vdim]
+  const float* norm = nullptr;     // [heads vdim]
+  int heads = 0, dim = 0, vdim = 0;
+  float q_scale = 1.f, gate_cap = 0.f, eps = 0.f;
+  float* state = nullptr;
+  long long slot_floats = 0;
+  int in_width() const { return 2 * heads * dim + 2 * heads * vdim + 2 * heads; }
+};
+void mlstm(Launch& l, const void* x, int m, int hidden, const MlstmArgs& a,
+           const mk_step_view& step, float* h, const float*& pending, int& pending_count);
 
 // act = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, k].  tile_config: -2 by the
 // sizes, else the tiled kernel with that configuration (-1: its own choice).
@@ -310,7 +342,7 @@ void* linear_per_head(Launch& l, const void* x, int m, int heads, int lda, int x
 // more as the value; a query head h scores (W_uk[h]^T q_h) . c + rot(q_rot_h) . r, and its
 // output is W_uv[h] applied to the attention's weighted sum of latents.
 struct LatentArgs {
-  const void* w_down = nullptr;    // [q_rank + kv_rank + rot, hidden]: query latent, c, r
+  const void* w_down = nullptr;    // [q_rank + kv_rank + rot + gate_cols, hidden]: query latent, c, r, gate
   const void *q_norm = nullptr, *kv_norm = nullptr;
   int norm_dtype = 0;
   float eps = 0.f;
@@ -318,6 +350,11 @@ struct LatentArgs {
   const void* w_uk_t = nullptr;    // [heads, kv_rank, dim]: W_uk per head, transposed
   const void* w_uv = nullptr;      // [heads, vdim, kv_rank]
   int heads = 0, dim = 0, rot = 0, vdim = 0, q_rank = 0, kv_rank = 0;
+  // q_rank 0: the queries come straight from the input, w_uq being [heads (dim + rot), hidden].
+  // gate_cols: further rows of w_down whose float32 products belong to the caller (a gate).
+  int gate_cols = 0;
+  int window = 0;                  // > 0: a query sees itself and the window - 1 tokens before it
+  const float* sinks = nullptr;    // [heads]: exp(sink) once more in the softmax's denominator
   PositionDesc pos;                // over the first pos.rotary_dim dims of the rotated parts
   void *k_cache = nullptr, *v_cache = nullptr;
   int page_size = 1;
@@ -336,8 +373,10 @@ struct LatentArgs {
 };
 // Down-projection, norms, rotation and cache write, query up-projection; the queries come back
 // as rows [heads, kv_rank + rot] = [absorbed | rotated].
+// `raw` / `raw_stride`, when not null, receive the float32 down-projection (the gate's
+// columns are its last gate_cols).
 Queries latent_queries(Launch& l, const void* x, int m, int hidden, const LatentArgs& a,
-                       const StepArrays& s);
+                       const StepArrays& s, const float** raw = nullptr, int* raw_stride = nullptr);
 // The attention over the cached latents: [m, heads, value_width()] weighted sums of them.
 struct LatentPlan {
   bool mfma = false;

@@ -4,7 +4,8 @@
 //   mk_retention_scan   S_t = decay S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head, the state
 //                       carried per request slot; queries and keys turn by their positions and
 //                       the keys are scaled on the way in;
-//   mk_head_norm_gate   a norm per head without a weight, then a gate of one number per column.
+//   mk_head_norm_gate   a norm per head, with or without a weight, then a gate of one number
+//                       per column (silu or sigmoid).
 //
 // The recurrence.  A workgroup of four wavefronts owns 32 columns of one head of one sequence;
 // a wavefront 8 of them by 8 slices of the state's rows, a lane one column and R = ceil(dim / 8)
@@ -214,7 +215,8 @@ __global__ __launch_bounds__(256) void retention_carry_kernel(
 template <typename T>
 __global__ __launch_bounds__(64) void head_norm_gate_kernel(
     const float* __restrict__ y, T* __restrict__ out, const float* __restrict__ gate,
-    int gate_stride, float eps, int heads, int dv) {
+    int gate_stride, float eps, int heads, int dv, const float* __restrict__ weight,
+    int gate_kind) {
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const float* row = y + ((size_t)t * heads + head) * dv;
   float sq = 0.f;
@@ -222,9 +224,10 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(
   const float r = rsqrtf(wave_sum(sq) / (float)dv + eps);
   for (int i = lane; i < dv; i += MK_WAVE) {
     float v = row[i] * r;
+    if (weight) v *= weight[head * dv + i];
     if (gate) {
       const float z = gate[(size_t)t * gate_stride + head * dv + i];
-      v *= z / (1.f + expf(-z));
+      v *= (gate_kind == MK_GATE_SIGMOID ? 1.f : z) / (1.f + expf(-z));
     }
     Elem<T>::store(out + ((size_t)t * heads + head) * dv + i, v);
   }
@@ -300,17 +303,19 @@ extern "C" long long mk_retention_scan_workspace(int total_chunks, int heads, in
 
 extern "C" int mk_head_norm_gate(const float* y, void* out, int dtype, const float* gate,
                                  int gate_stride, float eps, int tokens, int heads, int dv,
-                                 hipStream_t stream) {
+                                 const float* weight, int gate_kind, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && heads > 0 && dv > 0, "head_norm_gate: bad sizes");
+  MK_REQUIRE(gate_kind == MK_GATE_SILU || gate_kind == MK_GATE_SIGMOID,
+             "head_norm_gate: unknown gate %d", gate_kind);
   MK_REQUIRE(heads <= 65535, "head_norm_gate: too many heads (%d)", heads);
   MK_REQUIRE(!gate || gate_stride >= heads * dv, "head_norm_gate: gate rows of %d for %d columns",
              gate_stride, heads * dv);
   if (tokens == 0) return 0;
   const dim3 grid(tokens, heads);
   if (dtype == MK_F32)
-    head_norm_gate_kernel<float><<<grid, MK_WAVE, 0, stream>>>(y, (float*)out, gate, gate_stride, eps, heads, dv);
+    head_norm_gate_kernel<float><<<grid, MK_WAVE, 0, stream>>>(y, (float*)out, gate, gate_stride, eps, heads, dv, weight, gate_kind);
   else if (dtype == MK_BF16)
-    head_norm_gate_kernel<bf16_t><<<grid, MK_WAVE, 0, stream>>>(y, (bf16_t*)out, gate, gate_stride, eps, heads, dv);
+    head_norm_gate_kernel<bf16_t><<<grid, MK_WAVE, 0, stream>>>(y, (bf16_t*)out, gate, gate_stride, eps, heads, dv, weight, gate_kind);
   else
     MK_REQUIRE(false, "head_norm_gate: unknown dtype %d", dtype);
   MK_LAUNCH_CHECK("head_norm_gate");

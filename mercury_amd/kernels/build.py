@@ -36,6 +36,7 @@ LIBRARIES = {
         "mixers.hip",
         "state_space.hip",
         "retention.hip",
+        "mlstm.hip",
         "sampling.hip",
         "random_fill.hip",
     ],

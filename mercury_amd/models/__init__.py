@@ -1,3 +1,3 @@
 """Built-in architectures; importing this package registers them."""
 
-from . import larozen, qwen2, talolorn, videdra  # noqa: F401
+from . import larozen, mogilorn, qwen2, talolorn, videdra  # noqa: F401

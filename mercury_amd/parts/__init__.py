@@ -11,7 +11,8 @@ from .latent_attention import LatentAttention
 from .lowering import OneOp
 from .mixer_sum import NormedMixerSum
 from .model import CallerStep, DecoderModel, LayerCall, Registers
-from .norm import RMSNorm
+from .mlstm import MatrixMemory
+from .norm import NoNorm, RMSNorm
 from .position import NoPosition, RotaryPosition
 from .state_space import StateSpaceMixer
 from .stream_mix import StreamMix
@@ -27,7 +28,9 @@ register_ffn("unary_mlp")(UnaryMLP)
 register_mixer("state_space")(StateSpaceMixer)
 register_mixer("normed_sum")(NormedMixerSum)
 register_mixer("retention")(Retention)
+register_mixer("matrix_memory")(MatrixMemory)
 register_norm("rmsnorm")(RMSNorm)
+register_norm("none")(NoNorm)
 register_position("rotary")(RotaryPosition)
 register_position("none")(NoPosition)
 register_block("pre_norm")(PreNormBlock)
@@ -36,7 +39,7 @@ register_block("pre_post_norm")(PrePostNormBlock)
 
 __all__ = [
     "Attention", "CacheSpec", "CallerStep", "DecoderModel", "FeedForward", "GatedMLP",
-    "LatentAttention", "LayerCache", "LayerCall", "Mixer", "NoPosition", "Norm", "OneOp", "OutputHead", "Part",
+    "LatentAttention", "LayerCache", "LayerCall", "MatrixMemory", "Mixer", "NoNorm", "NoPosition", "Norm", "OneOp", "OutputHead", "Part",
     "ParallelBlock", "PositionDescriptor", "PrePostNormBlock", "Retention", "PositionEncoding", "PreNormBlock", "Registers",
     "RoutedExperts", "NormedMixerSum", "StateSpaceMixer", "StreamMix", "UnaryMLP",
     "RMSNorm", "RotaryPosition", "StateSpec", "TensorSpec", "TokenEmbedding", "build_part", "known",

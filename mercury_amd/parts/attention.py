@@ -13,7 +13,10 @@ from .lowering import OneOp
 # checkpoints call them otherwise passes its own map.
 DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj",
                  "q_norm": "q_norm", "k_norm": "k_norm", "sink": "sink", "gate": "g_proj",
-                 "lq1": "lambda_q1", "lk1": "lambda_k1", "lq2": "lambda_q2", "lk2": "lambda_k2"}
+                 "lq1": "lambda_q1", "lk1": "lambda_k1", "lq2": "lambda_q2", "lk2": "lambda_k2",
+                 "v_mix": "v_mix"}
+# the kernels' codes of `v_mix`
+V_MIX_CODES = {None: 0, "leave": 1, "blend": 2}
 
 
 class Attention(Mixer):
@@ -34,7 +37,9 @@ class Attention(Mixer):
     bias), before any norm or rotation.  `value_dim`: values of another width than the keys.
     `qk_norm` ("whole"): an RMS norm over the whole q projection and one over the whole k
     projection (all heads at once; plain weights ``<q_norm>.weight`` [n_q d] and
-    ``<k_norm>.weight`` [n_kv d], eps `norm_eps`), before the rotation.
+    ``<k_norm>.weight`` [n_kv d], eps `norm_eps`), before the rotation; ("head"): the norm runs
+    over every head by itself, with one weight of d entries for the query heads and one for the
+    key heads.
     `q_temp=(coef, every)`: the query at position p is multiplied by
     1 + coef * ln(floor((p + 1) / every) + 1), after its norm.
     `sinks`: a stored number per query head (``<sink>.weight`` [n_q]) whose exponential stands
@@ -55,6 +60,16 @@ class Attention(Mixer):
     the output projection.
     `own_kv=False`: the layer has no key and value projections; it reads a cache slot that
     another layer writes (whose head counts, widths and rotation are its own).
+    `out_gate`: a projection ``<gate>.weight`` [n_q value_dim, hidden] of the mixer's input whose
+    sigmoid multiplies the heads' outputs side by side, column by column, before the output
+    projection.
+    `v_mix`: values mixed across layers.  ``"leave"``: the layer's values of a step's tokens, as
+    projected, stay at hand for the layers after it; ``"blend"``: the layer caches and attends
+    over (1 - lam) v + lam v_left, v_left being what a "leave" layer earlier in the execution
+    list left for the same token and lam the stored number ``<v_mix>`` (a "leave" layer stores
+    one too and does not use it; `v_mix_stored` says whether a layer that does not mix stores
+    the number all the same: "yes", "maybe", "no").  Both kinds of layer have n_kv value_dim
+    value columns alike.
     """
 
     graph_safe = True   # forward launches kernels only: a decode step may be captured in a graph
@@ -68,7 +83,8 @@ class Attention(Mixer):
                  q_temp: tuple | None = None, sinks: bool = False, keep_first: int = 0,
                  maps: int = 1, diff_init: float = 0.0, head_gate: bool = False,
                  cache_window: int | None = -1, cache_keep_first: int | None = None,
-                 own_kv: bool = True):
+                 own_kv: bool = True, out_gate: bool = False, v_mix: str | None = None,
+                 v_mix_stored: str | None = None):
         if n_q % n_kv:
             raise ValueError(f"{n_q} query heads are not a multiple of {n_kv} key/value heads")
         self.hidden, self.n_q, self.n_kv, self.head_dim = int(hidden), int(n_q), int(n_kv), int(head_dim)
@@ -83,8 +99,8 @@ class Attention(Mixer):
         self.value_dim = int(value_dim) if value_dim else self.head_dim
         if self.values_are_keys and self.value_dim != self.head_dim:
             raise ValueError("values that are the keys are as wide as the keys")
-        if qk_norm not in (None, "whole"):
-            raise ValueError(f"qk_norm {qk_norm!r}: None or 'whole'")
+        if qk_norm not in (None, "whole", "head"):
+            raise ValueError(f"qk_norm {qk_norm!r}: None, 'whole' or 'head'")
         self.qk_norm, self.norm_eps = qk_norm, float(norm_eps)
         self.q_temp = (float(q_temp[0]), int(q_temp[1])) if q_temp else None
         if self.q_temp and self.q_temp[1] <= 0:
@@ -107,6 +123,20 @@ class Attention(Mixer):
         self.diff_lambda = 0.0
         self.w_q_gate = None
         self.own_kv = bool(own_kv)
+        self.out_gate = bool(out_gate)
+        if self.out_gate and (self.head_gate or self.maps > 1 or not self.own_kv):
+            raise ValueError("a gate per column goes with one map a head, no gate per head, and "
+                             "a layer's own keys and values")
+        if v_mix not in V_MIX_CODES:
+            raise ValueError(f"v_mix {v_mix!r}: None, 'leave' or 'blend'")
+        self.v_mix = v_mix
+        if self.v_mix and (self.values_are_keys or not self.own_kv or self.maps > 1):
+            raise ValueError("values mixed across layers are a layer's own projected values")
+        self.v_lambda = 0.0
+        # whether the number is stored: "yes", "maybe" (loaded when there, never used), "no"
+        self.v_mix_stored = v_mix_stored or ("yes" if self.v_mix else "no")
+        if self.v_mix_stored not in ("yes", "maybe", "no") or (self.v_mix and self.v_mix_stored != "yes"):
+            raise ValueError("v_mix_stored: 'yes', 'maybe' or 'no'; a layer that mixes stores its number")
         if not self.own_kv and self.values_are_keys:
             raise ValueError("values that are keys are a layer's own")
         self.names = {**DEFAULT_NAMES, **(names or {})}
@@ -119,7 +149,8 @@ class Attention(Mixer):
         """Whether q and k get more than a rotation between projection and cache (the kernels
         then take the projection in float32 and do all of it in one pass)."""
         return bool(self.values_are_keys or self.qk_norm or self.q_temp
-                    or self.value_dim != self.head_dim or self.maps > 1)
+                    or self.value_dim != self.head_dim or self.maps > 1 or self.out_gate
+                    or self.v_mix)
 
     # ---- declarations
 
@@ -149,10 +180,15 @@ class Attention(Mixer):
         if self.o_bias:
             specs[f"{n['o']}.bias"] = TensorSpec((h,), role="vector")
         if self.qk_norm:
-            specs[f"{n['q_norm']}.weight"] = TensorSpec((self.n_q * self.head_dim,), role="vector",
-                                                        init="one_plus_normal")
-            specs[f"{n['k_norm']}.weight"] = TensorSpec((self.n_kv * self.head_dim,), role="vector",
-                                                        init="one_plus_normal")
+            per = 1 if self.qk_norm == "head" else None
+            specs[f"{n['q_norm']}.weight"] = TensorSpec(((per or self.n_q) * self.head_dim,),
+                                                        role="vector", init="one_plus_normal")
+            specs[f"{n['k_norm']}.weight"] = TensorSpec(((per or self.n_kv) * self.head_dim,),
+                                                        role="vector", init="one_plus_normal")
+        if self.out_gate:
+            specs[f"{n['gate']}.weight"] = TensorSpec((self.n_q * self.value_dim, h))
+        if self.v_mix_stored != "no":
+            specs[n["v_mix"]] = TensorSpec((), role="vector", optional=self.v_mix_stored == "maybe")
         if self.sinks:
             specs[f"{n['sink']}.weight"] = TensorSpec((self.n_q,), role="vector")
         if self.maps > 1:
@@ -173,7 +209,11 @@ class Attention(Mixer):
             gate = params[f"{n['gate']}.weight"]
             stacked.append(gate)
             self.w_q_gate = torch.cat([stacked[0], gate], dim=0).contiguous()
+        if self.out_gate:
+            stacked.append(params[f"{n['gate']}.weight"])
         self.w_qkv = torch.cat(stacked, dim=0).contiguous()
+        if self.v_mix:
+            self.v_lambda = float(params[n["v_mix"]].float())
         if self.maps > 1:
             dot = lambda a, b: (params[n[a]].float() * params[n[b]].float()).sum()
             self.diff_lambda = float(torch.exp(dot("lq1", "lk1")) - torch.exp(dot("lq2", "lk2"))
@@ -181,6 +221,9 @@ class Attention(Mixer):
         if self.qkv_bias:
             biases = [params[f"{n[key]}.bias"] for key in keys]
             common = torch.float32 if any(b.dtype == torch.float32 for b in biases) else dtype
+            if self.out_gate:     # the gate's rows have no bias
+                biases.append(torch.zeros(self.n_q * self.value_dim, dtype=common,
+                                          device=biases[0].device))
             self.b_qkv = torch.cat([b.to(common) for b in biases]).contiguous()
         self.w_o = params[f"{n['o']}.weight"]
         self.b_o = params.get(f"{n['o']}.bias")
@@ -229,6 +272,11 @@ class Attention(Mixer):
             w, b = w[:rows], None if b is None else b[:rows]
             if self.head_gate:
                 w = self.w_q_gate
+            if self.out_gate or self.v_mix:
+                raise ValueError("a gate per column and mixed values go with a cache the layer writes")
+        if self.v_mix:
+            # room in the step for what a "leave" layer hands to the "blend" layers after it
+            program.need_carried(self.n_kv * self.value_dim)
         # (a kind of its own where the fixed-point stream's kernels would not do the same)
         program.append("attention_prepared" if self.prepared or self.sinks else "attention",
                        core.attention_params(
@@ -248,7 +296,9 @@ class Attention(Mixer):
             value_dim=self.value_dim if self.prepared else 0,
             keep_first=self.keep_first, maps=self.maps, head_gate=self.head_gate,
             diff_lambda=self.diff_lambda, diff_eps=self.norm_eps,
-            diff_scale=1.0 - self.diff_init if self.maps > 1 else 1.0))
+            diff_scale=1.0 - self.diff_init if self.maps > 1 else 1.0,
+            head_norm=self.qk_norm == "head", out_gate=self.out_gate,
+            v_mode=V_MIX_CODES[self.v_mix], v_lambda=self.v_lambda))
 
     def forward(self, x, step, cache, state, accum):
         if self.position.describe() is not None:

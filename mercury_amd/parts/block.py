@@ -132,6 +132,8 @@ class PrePostNormBlock(Part):
     def _wrapped(self, program, sub: "_Recorder", post: Norm, scale) -> None:
         if len(sub.ops) != 1:
             raise ValueError("a sublayer between two norms lowers itself to one operation")
+        if getattr(sub, "carried", 0):
+            program.need_carried(sub.carried)
         if getattr(post, "one_plus", False) and post.weight is None:
             raise ValueError("the norm behind a sublayer has no weight yet")
         program.append("post_norm", core.post_norm_params(
@@ -205,6 +207,9 @@ class _Recorder:
     def append(self, kind: str, params: bytes) -> None:
         self.ops.append((kind, params))
 
+    def need_carried(self, width: int) -> None:
+        self.carried = max(getattr(self, "carried", 0), int(width))
+
 
 class ParallelBlock(Part):
     """h += mult * (mixer(x) + ffn(x)) with x = norm(h): one norm, both sublayers read its
@@ -250,6 +255,8 @@ class ParallelBlock(Part):
             self.ffn.lower(sub)
         if len(sub.ops) != (1 if self.ffn is None else 2):
             raise ValueError("a sublayer of a parallel block lowers itself to one operation")
+        if getattr(sub, "carried", 0):
+            program.need_carried(sub.carried)
         program.append("parallel", core.parallel_params(self.residual_mult, sub.ops))
 
     def param_specs(self) -> dict:

@@ -76,7 +76,7 @@ class GatedMLP(FeedForward):
         return pending
 
 
-UNARY_ACTIVATIONS = {"relu2": 0}     # the kernels' codes
+UNARY_ACTIVATIONS = {"relu2": 0, "gelu_tanh": 1}     # the kernels' codes
 UNARY_NAMES = {"up": "up_proj", "down": "down_proj"}
 
 
@@ -84,6 +84,7 @@ class UnaryMLP(FeedForward):
     """down(act(up(x))) without biases, for an activation of one operand.  `activation`:
 
     ``"relu2"``: the square of relu.
+    ``"gelu_tanh"``: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
 
     `names` maps up, down to the stored tensors' leaf names (default ``up_proj``,
     ``down_proj``)."""

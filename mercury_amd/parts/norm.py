@@ -8,6 +8,31 @@ from .base import Norm, TensorSpec
 from .lowering import OneOp
 
 
+class NoNorm(Norm):
+    """No norm at all: a sublayer that reads the residual stream itself.  y = x in the output
+    dtype (after the partial sums before it have been added into the stream)."""
+
+    graph_safe = True
+    lowerable = True
+
+    def __init__(self, size: int):
+        self.size = int(size)
+        self._alone = None
+
+    def forward(self, h, out_dtype, rows=None, partials=None):
+        if rows is not None:
+            raise ValueError("the stream as it stands is read whole")
+        if self._alone is None:
+            self._alone = OneOp(out_dtype, self.size, 0, self.lower)
+        _logits, x, _pending = self._alone.run(None, h, pending=partials)
+        return x
+
+    def lower(self, program, select_rows: bool = False) -> None:
+        if select_rows:
+            raise ValueError("the stream as it stands is read whole")
+        program.append("stream_cast", core.stream_cast_params())
+
+
 class RMSNorm(Norm):
     """y = (x * rsqrt(mean(x^2) + eps)) * weight, statistics in float32.
 

@@ -51,7 +51,9 @@ class OpContext(ctypes.Structure):
                 ("stream_fixed", c_int), ("h_fixed", c_void_p),
                 ("norm_weight", c_void_p), ("norm_weight_dtype", c_int), ("norm_eps", c_float),
                 ("out_norm_weight", c_void_p), ("out_norm_weight_dtype", c_int),
-                ("out_norm_eps", c_float), ("kept", POINTER(c_float))]
+                ("out_norm_eps", c_float), ("kept", POINTER(c_float)),
+                # float32 [T, carried_width] for values one operation leaves to later ones
+                ("carried", POINTER(c_float)), ("carried_width", c_int)]
 
     def allocate(self, nbytes: int) -> int:
         """Device memory from the operation's arena (0 in a dry walk)."""
