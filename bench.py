@@ -31,6 +31,12 @@ does the same for the Larozen design (rotated attention with a bounded score who
 its keys, alternating with layers of a sink attention beside a state-space mixer; squared-relu
 feed-forwards; one re-entry of the stream), and
 
+    python bench.py --mogilorn [--mogilorn-only NAME]
+
+for the Mogilorn design (a gated attention whose values are mixed across layers, a gated matrix
+memory, a windowed latent attention with sinks; sublayers that read the stream itself) beside
+Videdra and Qwen2, and
+
     python bench.py --shape 32b --serve
 
 runs a whole workload through the scheduler instead (64 requests with prompts of 2,048 tokens,
@@ -115,6 +121,13 @@ def parse_args(argv=None):
                         "layer sizes, beside Larozen and Qwen2 at equal width, depth and heads")
     p.add_argument("--videdra-only", default=None,
                    help="run one entry of the comparison only (e.g. small/videdra-moe), for a profiler")
+    p.add_argument("--mogilorn", action="store_true",
+                   help="prompts and decode steps of the Mogilorn design (gated attention with "
+                        "values mixed across layers, a gated matrix memory, a windowed latent "
+                        "attention with sinks) at two sets of layer sizes, beside Videdra and "
+                        "Qwen2 at equal width, depth and heads")
+    p.add_argument("--mogilorn-only", default=None,
+                   help="run one entry of the comparison only (e.g. small/mogilorn), for a profiler")
     p.add_argument("--serve-requests", type=int, default=64)
     p.add_argument("--serve-chunk", type=int, default=512)
     return p.parse_args(argv)
@@ -521,6 +534,37 @@ def videdra_configs(z: dict) -> dict:
             "larozen": others["larozen"], "qwen2": others["qwen2"]}
 
 
+# Layer sizes for `--mogilorn`: four layers (an attention that leaves its values, a matrix
+# memory, a latent attention in a window of 1,024, an attention that blends the first one's
+# values in); heads of 128 over values of 128, memory heads of 64 x 128, a latent of 512 with a
+# turned part of 64.
+MOGILORN_SIZES = {
+    size: dict(z, kv_rank=512, rot_dim=64, mem_heads=z["ret_heads"], mem_dim=z["ret_dim"],
+               mem_vdim=z["ret_vdim"])
+    for size, z in VIDEDRA_SIZES.items()
+}
+
+
+def mogilorn_configs(z: dict) -> dict:
+    """name -> config.json of the three models compared at the sizes `z`."""
+    attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                 "scale": z["dim"] ** -0.5, "softcap": 30.0, "v_mix": True,
+                 "rot": {"base": 10000.0, "dims": z["dim"],
+                         "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    memory = {"heads": z["mem_heads"], "dim": z["mem_dim"], "vdim": z["mem_vdim"], "gate_cap": 15.0}
+    latent = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["dim"],
+              "kv_rank": z["kv_rank"], "scale": (z["dim"] + z["rot_dim"]) ** -0.5,
+              "mask": {"size": z["window"]}, "rot": {"base": 10000.0, "dims": z["rot_dim"]}}
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    kinds = [("attention", attention), ("mlstm", memory), ("latent_attention", latent),
+             ("attention", attention)]
+    others = videdra_configs(z)
+    return {"mogilorn": {"architecture": "Mogilorn", "vocab": z["vocab"], "width": z["width"],
+                         "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+                         "layers": [{"type": kind, "mixer": mixer, "mlp": mlp} for kind, mixer in kinds]},
+            "videdra": others["videdra-dense"], "qwen2": others["qwen2"]}
+
+
 def talolorn_main(args) -> int:
     return compare_main(args, "Talolorn", TALOLORN_SIZES, talolorn_configs, args.talolorn_only)
 
@@ -531,6 +575,10 @@ def larozen_main(args) -> int:
 
 def videdra_main(args) -> int:
     return compare_main(args, "Videdra", VIDEDRA_SIZES, videdra_configs, args.videdra_only)
+
+
+def mogilorn_main(args) -> int:
+    return compare_main(args, "Mogilorn", MOGILORN_SIZES, mogilorn_configs, args.mogilorn_only)
 
 
 def compare_main(args, design: str, sizes: dict, configs, only) -> int:
@@ -579,6 +627,8 @@ def main(argv=None) -> int:
         return larozen_main(args)
     if args.videdra:
         return videdra_main(args)
+    if args.mogilorn:
+        return mogilorn_main(args)
     model_name, shape = SHAPES[args.shape]
     cfg = dict(shape)
     full_layers = cfg["num_hidden_layers"]

@@ -20,6 +20,11 @@
 // before its first product.  With the keys split into parts, every part leaves an
 // unnormalised result with its running maximum and sum, and a second kernel merges the parts
 // in order.
+//
+// With a window a row sees the keys (pos - window, pos]: a tile starts at the block of the
+// first key any of its rows sees, and the lower edge is masked like the upper one.  With
+// sinks a head's exp(sink) is added to the denominator of its rows where the result is
+// normalised (here, or in the merge of the parts).
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -51,7 +56,11 @@ struct LatentAttnParams {
   int num_tiles;
   int num_parts;
   int dvt;               // for the merge kernel
+  int window;            // > 0: a row at position p sees keys (p - window, p] only
+  const float* sinks;    // [heads] or null: exp(sink) once more in a row's denominator
 };
+
+#define LOG2E 1.4426950408889634f
 
 #define LAT_WAVES 4
 
@@ -93,8 +102,12 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 1 : 2)) void attn_la
   const int kmax = kv_len - q_len + last_row / p.heads;       // the tile's last visible key
   const int all_see = kv_len - q_len + row0 / p.heads;         // keys every row of it sees
   const int blocks = (kmax >> 5) + 1;
-  const int per = (blocks + p.num_parts - 1) / p.num_parts;
-  const int b_begin = part * per, b_end = min(blocks, b_begin + per);
+  // the first key any row sees, and the first one all of them see
+  const int lo_any = p.window > 0 ? max(0, all_see - p.window + 1) : 0;
+  const int lo_all = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
+  const int b_first = lo_any >> 5;
+  const int per = (blocks - b_first + p.num_parts - 1) / p.num_parts;
+  const int b_begin = b_first + part * per, b_end = min(blocks, b_begin + per);
   const int ps = 1 << p.page_shift;
   constexpr int DK = DKC * 32, DV = DVT * 16;
   const int* table = p.block_table + (size_t)seq * p.table_stride;
@@ -185,6 +198,13 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 1 : 2)) void attn_la
         for (int i = 0; i < 4; ++i)
           if (key0 + h * 16 + g4 * 4 + i > pos) s[h * 4 + i] = -INFINITY;
     }
+    if (key0 < lo_all) {         // keys the window of some row has passed
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (key0 + h * 16 + g4 * 4 + i <= pos - p.window) s[h * 4 + i] = -INFINITY;
+    }
     float bm = c2 * fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
                           fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
     if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
@@ -232,6 +252,7 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 1 : 2)) void attn_la
 
   if (p.num_parts == 1) {
     if (!row_ok) return;
+    if (p.sinks) lsum += __builtin_amdgcn_exp2f(p.sinks[head] * LOG2E - m);
     const float inv = 1.f / lsum;
     bf16_t* dst = p.out + ((size_t)token * p.heads + head) * DV + g4 * 4;
 #pragma unroll
@@ -279,8 +300,12 @@ __global__ __launch_bounds__(256) void attn_latent_split_values_kernel(LatentAtt
   const int kmax = kv_len - q_len + last_row / p.heads;
   const int all_see = kv_len - q_len + row0 / p.heads;
   const int blocks = (kmax >> 5) + 1;
-  const int per = (blocks + p.num_parts - 1) / p.num_parts;
-  const int b_begin = part * per, b_end = min(blocks, b_begin + per);
+  // the first key any row sees, and the first one all of them see
+  const int lo_any = p.window > 0 ? max(0, all_see - p.window + 1) : 0;
+  const int lo_all = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
+  const int b_first = lo_any >> 5;
+  const int per = (blocks - b_first + p.num_parts - 1) / p.num_parts;
+  const int b_begin = b_first + part * per, b_end = min(blocks, b_begin + per);
   const int ps = 1 << p.page_shift;
   constexpr int DK = DKC * 32, DV = DVT * 16;
   const int* table = p.block_table + (size_t)seq * p.table_stride;
@@ -337,6 +362,13 @@ __global__ __launch_bounds__(256) void attn_latent_split_values_kernel(LatentAtt
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (key0 + h * 16 + g4 * 4 + i > pos) s[h * 4 + i] = -INFINITY;
+    }
+    if (key0 < lo_all) {         // keys the window of some row has passed
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (key0 + h * 16 + g4 * 4 + i <= pos - p.window) s[h * 4 + i] = -INFINITY;
     }
     float bm = c2 * fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
                           fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
@@ -406,6 +438,11 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 2 : 1)) void attn_la
   const int my_kmax = first_pos + min(my_row0 + 15, rows - 1) / p.heads;
   const int all_see = first_pos + min(my_row0, rows - 1) / p.heads;
   const int blocks = ((first_pos + min(row0 + 63, rows - 1) / p.heads) >> 5) + 1;
+  // with a window: the first key any row of the wavefront sees, the first all of them see, and
+  // the block the workgroup's walk starts at
+  const int lo_any = p.window > 0 ? max(0, all_see - p.window + 1) : 0;
+  const int lo_all = p.window > 0 ? max(0, my_kmax - p.window + 1) : 0;
+  const int b_first = p.window > 0 ? max(0, first_pos + row0 / p.heads - p.window + 1) >> 5 : 0;
   const int ps = 1 << p.page_shift;
   const int* table = p.block_table + (size_t)seq * p.table_stride;
 
@@ -423,7 +460,7 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 2 : 1)) void attn_la
   constexpr int K_CHUNKS = 32 * (DK / 8), V_CHUNKS = DV * 4;   // 16-byte pieces of a block
   constexpr int K_MINE = (K_CHUNKS + 255) / 256, V_MINE = (V_CHUNKS + 255) / 256;
 
-  for (int b = 0; b < blocks; ++b) {
+  for (int b = b_first; b < blocks; ++b) {
     const int key0 = b << 5;
     // the two halves' places in the cache (scalars: an array indexed by the half would live
     // in scratch memory)
@@ -491,7 +528,7 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 2 : 1)) void attn_la
 #undef LAT_V_FROM
 #undef LAT_V_TO
     __syncthreads();
-    if (!wave_live || key0 > my_kmax) continue;      // the wavefront's rows see nothing here
+    if (!wave_live || key0 > my_kmax || key0 + 31 < lo_any) continue;   // the wavefront's rows see nothing here
     float s[8];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -511,6 +548,13 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 2 : 1)) void attn_la
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (key0 + h * 16 + g4 * 4 + i > pos) s[h * 4 + i] = -INFINITY;
+    }
+    if (key0 < lo_all) {         // keys the window of some row has passed
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (key0 + h * 16 + g4 * 4 + i <= pos - p.window) s[h * 4 + i] = -INFINITY;
     }
     float bm = c2 * fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
                           fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
@@ -543,6 +587,7 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 2 : 1)) void attn_la
   if (!row_ok) return;
   lsum += __shfl_xor(lsum, 16, 64);
   lsum += __shfl_xor(lsum, 32, 64);
+  if (p.sinks) lsum += __builtin_amdgcn_exp2f(p.sinks[head] * LOG2E - m);
   const float inv = 1.f / lsum;
   bf16_t* dst = p.out + ((size_t)token * p.heads + head) * DV + g4 * 4;
 #pragma unroll
@@ -557,7 +602,7 @@ __global__ __launch_bounds__(256, (latent_early(DKC, DVT) ? 2 : 1)) void attn_la
 // rows, in part order.
 __global__ __launch_bounds__(256) void attn_latent_merge_kernel(LatentAttnParams p) {
   __shared__ float weight[LATENT_MAX_PARTS][16];
-  __shared__ float inv[16];
+  __shared__ float inv[16], top[16];
   const int tile = blockIdx.x;
   const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
@@ -573,6 +618,7 @@ __global__ __launch_bounds__(256) void attn_latent_merge_kernel(LatentAttnParams
     float m = -INFINITY;
     for (int s = 0; s < p.num_parts; ++s) m = fmaxf(m, weight[s][r]);
     inv[r] = m;
+    top[r] = m;
   }
   __syncthreads();
   for (int i = threadIdx.x; i < p.num_parts * 16; i += blockDim.x) {
@@ -584,6 +630,9 @@ __global__ __launch_bounds__(256) void attn_latent_merge_kernel(LatentAttnParams
     const int r = threadIdx.x;
     float total = 0.f;
     for (int s = 0; s < p.num_parts; ++s) total += weight[s][r] * ml[s * 32 + 16 + r];
+    if (p.sinks && row0 + r < rows) {
+      total += __builtin_amdgcn_exp2f(p.sinks[(row0 + r) % p.heads] * LOG2E - top[r]);
+    }
     inv[r] = 1.f / total;
   }
   __syncthreads();
@@ -649,7 +698,9 @@ extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache
                                    int num_tiles, int tile_rows, const int* cu_q, const int* kv_len,
                                    const int* block_table, int table_stride, int page_size,
                                    int heads, int dk, int dv, float scale, int num_parts,
-                                   float* part_o, float* part_ml, hipStream_t stream) {
+                                   float* part_o, float* part_ml, int window, const float* sinks,
+                                   hipStream_t stream) {
+  MK_REQUIRE(window >= 0, "latent attention: negative window");
   MK_REQUIRE(tile_rows == 16 || (tile_rows == 64 && num_parts == 1),
              "latent attention: tiles of 16 rows, or of 64 with the keys unsplit");
   MK_REQUIRE(mk_attention_latent_supported(dk, dv, page_size),
@@ -681,6 +732,8 @@ extern "C" int mk_attention_latent(const void* q, void* out, const void* k_cache
   p.num_tiles = num_tiles;
   p.num_parts = num_parts;
   p.dvt = dv / 16;
+  p.window = window;
+  p.sinks = sinks;
   const long long units = (long long)num_tiles * num_parts;
   // few units: one wavefront a workgroup, so that they spread over the compute units
   const int waves = units >= 2048 ? LAT_WAVES : 1;

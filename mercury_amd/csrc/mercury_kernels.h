@@ -437,7 +437,9 @@ int mk_expert_down_mfma(const void* act, const void* w, float* y, const int* row
 // that many parts (at most mk_attention_latent_max_parts()) whose results part_o
 // [tiles, parts, dv, 16] / part_ml [tiles, parts, 2, 16] a second kernel merges.  tile_rows 64
 // (keys unsplit): tiles of 64 rows, one a workgroup, whose wavefronts share every block of
-// keys through LDS: for prompt portions.  No window.
+// keys through LDS: for prompt portions.  window > 0: a row at position p sees the keys
+// (p - window, p] only.  sinks (float32 [heads], or null): exp(sink[head]) stands once more in
+// the denominator of the head's rows, unscaled.
 // Key and value widths come from a list of compiled shapes: mk_attention_latent_widths gives
 // the widths a cache must have for keys of at least dk and values of at least dv dims (host
 // pointers; returns 0 when no shape holds them), padded with zeros.
@@ -449,7 +451,7 @@ int mk_attention_latent(const void* q, void* out, const void* k_cache, const voi
                         const int* cu_q,
                         const int* kv_len, const int* block_table, int table_stride, int page_size,
                         int heads, int dk, int dv, float scale, int num_parts, float* part_o,
-                        float* part_ml, hipStream_t stream);
+                        float* part_ml, int window, const float* sinks, hipStream_t stream);
 
 // y = x W^T (+ bias) for any M, tiled through LDS; output bfloat16 or float32, or float32
 // accumulated into `out`.  config: a tile configuration, 0 .. mk_linear_tiled_configs() - 1

@@ -762,14 +762,14 @@ constexpr int kLatentMinBlocks = 4;
 LatentPlan latent_plan(int dtype, const LatentArgs& a, const mk_step_view& step) {
   LatentPlan plan;
   if (dtype != kBF16 || !kernels().has_mfma()) return plan;
-  // a window or sinks: the float32-arithmetic kernel
-  if (a.window > 0 || a.sinks != nullptr) return plan;
   const KernelTable& t = need_mfma();
   if (!t.mk_attention_latent_supported(a.key_width(), a.value_width(), a.page_size)) return plan;
   plan.mfma = true;
   const std::vector<int> counts(step.counts, step.counts + step.num_seqs);
   plan.num_tiles = count_tiles(counts, a.heads, 16);
-  const int blocks = (step.max_kv_len + 31) / 32;
+  // (inside a window a tile walks the window's blocks and one more, whatever the length)
+  const int reach = a.window > 0 ? std::min(step.max_kv_len, a.window + 31) : step.max_kv_len;
+  const int blocks = (reach + 31) / 32;
   int parts = 1;
   if (plan.num_tiles > 0 && plan.num_tiles < kLatentWaves) {
     parts = std::min(kLatentWaves / plan.num_tiles, std::max(1, blocks / kLatentMinBlocks));
@@ -809,7 +809,8 @@ void* latent_attend(Launch& l, const Queries& q, const LatentArgs& a, float scal
                                              tiles.count, plan.tile_rows, s.cu_q, s.kv_len, s.table,
                                              s.table_stride,
                                              a.page_size, a.heads, dk, dv, scale, plan.parts, part_o,
-                                             part_ml, l.stream()), "latent_attention");
+                                             part_ml, a.window, a.sinks, l.stream()),
+             "latent_attention");
   return out;
 }
 

@@ -340,6 +340,33 @@ def test_the_edge_of_the_window_shows(dtype, window):
 
 
 @pytest.mark.parametrize("dtype", BOTH)
+@pytest.mark.parametrize("window", [0, 300])
+def test_decoding_over_many_latents_splits_them_over_wavefronts(dtype, window):
+    """A prompt of 700 tokens, then 40 decoded one by one: a decoding step's keys (all 700 and
+    more, or the 300 of the window) are walked in parts that a second kernel merges, sinks
+    included; sharpened queries put weight on keys hundreds of tokens back."""
+    hidden = 64
+    m = latent(4, 8, 8, 16, 24, 0.5, window=window, rot=(1000.0, 8))
+    part = windowed_latent(hidden, m)
+    params = bind_random(part, dtype, scale=0.25, seed=43)
+    rebind(part, params, dtype, lambda p: (p["q.weight"].mul_(5.0), p["sink.weight"].add_(1.0)))
+    total = 740
+    x = rnd(total, hidden, seed=15).to(dtype).float()
+    cuts = [(0, 700)] + [(700 + i, 1) for i in range(40)]
+    got = run_mixer_in_portions(part, x.to(dtype), dtype, hidden, pages=48, portions=cuts)
+    positions = torch.arange(total)
+
+    def run(to, r):
+        w = {n: to(t) for n, t in plain_names(params).items()}
+        return plain.latent_attention(to(x), w, "p.", m, 1e-5, positions, r)
+
+    want = compare(got, run, dtype, slack=2.0)
+    w = plain_names(params)
+    nearer = dict(m, mask={"size": 200})
+    assert (plain.latent_attention(x, w, "p.", nearer, 1e-5, positions)[-40:] - want[-40:]).abs().max() > 0.01
+
+
+@pytest.mark.parametrize("dtype", BOTH)
 def test_keys_far_back_and_at_page_borders(dtype):
     """The gated attention with its score bounded loosely and queries scaled up: the softmax
     sits on single keys hundreds of tokens back; 600 tokens whole, then decoded across page
