@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 36
+#define MK_ABI_VERSION 37
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit);
@@ -336,11 +336,17 @@ int mk_head_norm_gate(const float* y, void* out, int dtype, const float* gate, i
 // (gate_cap <= 0: no bound).  A sequence's state is its slot's row of `state`
 // (mk_mlstm_state_floats(...) floats, rows slot_stride apart), read at the step's start and left
 // for the next; out [T, heads vdim] float32.
+// total_chunks > 0: every sequence runs as ceil(tokens / mk_mlstm_chunk_tokens()) chunks side by
+// side (total_chunks of them in the step) over a workspace of mk_mlstm_scan_workspace(...)
+// floats; 0: token by token from the slot's state.
 long long mk_mlstm_state_floats(int heads, int dim, int vdim);
+int mk_mlstm_chunk_tokens(void);
+long long mk_mlstm_scan_workspace(int total_chunks, int tokens, int heads, int dim, int vdim);
 int mk_mlstm_scan(const float* proj, int proj_stride, int q_col, int k_col, int v_col, int i_col,
                   int f_col, float q_scale, float gate_cap, const int* cu_q, const int* slots,
                   float* state, long long slot_stride, int heads, int dim, int vdim, float* out,
-                  int tokens, int num_seqs, hipStream_t stream);
+                  int tokens, int num_seqs, int total_chunks, float* workspace,
+                  hipStream_t stream);
 // out[t, part] = y[t, part] / rms(y[t, part]) * weight[part], the row in `parts` equal parts.
 int mk_group_rmsnorm(const float* y, void* out, int dtype, const void* weight, int weight_dtype,
                      float eps, int tokens, int width, int parts, hipStream_t stream);

@@ -21,6 +21,22 @@
 // tokens up to its own in the sequence's order, so that m, and with it every sum, is the same
 // however the sequence was cut into steps and whatever else the step holds.
 //
+// A step with a sequence longer than ML_CHUNK tokens runs in chunks side by side.  With
+// b_j the sum of the log forget gates from the chunk's first token to its j-th, m the running
+// maximum of the whole sequence and m' the one of the chunk alone (from minus infinity):
+//   gates     one wavefront a (sequence, head) walks the gates in order and leaves, per token,
+//             the chunk's own recurrence weights exp(f_j + m'_(j-1) - m'_j), exp(i_j - m'_j),
+//             the weights w1 = exp(b_j + m_start - m_j), w2 = exp(m'_j - m_j) that put the
+//             chunk's start state and its own part together, and exp(-m_j); per chunk the
+//             same two weights at its last token; and the slot's new m;
+//   pass 1    every chunk's recurrence from a zero state under m' (its numerators and n . q
+//             into `out` and a side buffer, its last state into the workspace);
+//   carry     the chunks' start states one after the other,
+//             S_start(c + 1) = w1_end(c) S_start(c) + w2_end(c) S_own(c), the last into the slot;
+//   pass 2    S_start^T q_j of every token, and w1 (that) + w2 (pass 1's) over the floored
+//             denominator.
+// Every exponent above is at most zero: m_j >= b_j + m_start and m_j >= m'_j.
+//
 // A slot holds [heads, dim, vdim] floats of S, then n [heads, B, dim] and m [heads, B] once for
 // each of the B = ceil(vdim / 28) workgroups of a head: a workgroup reads and writes a copy of
 // its own (the copies are equal, made by the same operations in the same order), so none reads
@@ -32,6 +48,8 @@
 #define ML_WAVE_COLUMNS 7  // columns of S a wavefront owns beside its copy of n
 #define ML_COLUMNS 28      // columns of a head per workgroup
 #define ML_MAX_DIM 256
+#define ML_CHUNK 128       // tokens of a chunk when a step runs in chunks
+#define ML_GATE_FIELDS 5   // per (token, head): keep', take', w1, w2, exp(-m)
 
 namespace {
 
@@ -40,47 +58,161 @@ __device__ __forceinline__ float log_sigmoid(float z) {
   return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
 }
 
-template <int R>
+__device__ __forceinline__ void activated_gates(const float* __restrict__ row, int i_col, int f_col,
+                                                int head, float gate_cap, float& log_in,
+                                                float& log_keep) {
+  float a = row[i_col + head], b = row[f_col + head];
+  if (gate_cap > 0.f) {
+    a = gate_cap * tanhf(a / gate_cap);
+    b = gate_cap * tanhf(b / gate_cap);
+  }
+  log_in = a;
+  log_keep = log_sigmoid(b);
+}
+
+// The sequence and the tokens of chunk `c` of the step.
+__device__ __forceinline__ void chunk_span(const int* __restrict__ cu_q, int num_seqs, int c,
+                                           int& seq, int& t_begin, int& t_end) {
+  int first = 0;
+  for (seq = 0; seq < num_seqs; ++seq) {
+    const int n = (cu_q[seq + 1] - cu_q[seq] + ML_CHUNK - 1) / ML_CHUNK;
+    if (c < first + n) break;
+    first += n;
+  }
+  if (seq >= num_seqs) {
+    t_begin = t_end = 0;
+    return;
+  }
+  t_begin = cu_q[seq] + (c - first) * ML_CHUNK;
+  t_end = min(cu_q[seq + 1], t_begin + ML_CHUNK);
+}
+
+// One wavefront a (sequence, head): the gates of the sequence's tokens in order.
+// gates [tokens, heads, ML_GATE_FIELDS]; ends [chunks, heads, 2] (w1 and w2 at a chunk's last
+// token); the slot's copies of m are read (the first) and written (all).
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(
+    const float* __restrict__ proj, int proj_stride, int i_col, int f_col, float gate_cap,
+    const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ state,
+    long long slot_stride, int heads, int dim, int vdim, int copies, float* __restrict__ gates,
+    float* __restrict__ ends) {
+  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int t_begin = cu_q[seq], t_end = cu_q[seq + 1];
+  if (t_begin >= t_end) return;
+  int chunk = 0;     // the sequence's first chunk among the step's
+  for (int i = 0; i < seq; ++i) chunk += (cu_q[i + 1] - cu_q[i] + ML_CHUNK - 1) / ML_CHUNK;
+  float* m_at = state + (size_t)slots[seq] * slot_stride + (size_t)heads * dim * vdim +
+                (size_t)heads * copies * dim + (size_t)head * copies;
+  float m = *m_at, own = -INFINITY, sum = 0.f, m_start = m;
+  for (int t0 = t_begin; t0 < t_end; t0 += MK_WAVE) {
+    const int count = min(MK_WAVE, t_end - t0);
+    float log_in = 0.f, log_keep = 0.f;
+    if (lane < count) {
+      activated_gates(proj + (size_t)(t0 + lane) * proj_stride, i_col, f_col, head, gate_cap,
+                      log_in, log_keep);
+    }
+    float my_m = 0.f, my_own = 0.f, my_own_before = 0.f, my_sum = 0.f, my_start = 0.f;
+    for (int j = 0; j < count; ++j) {
+      const float a = __shfl(log_in, j, MK_WAVE), b = __shfl(log_keep, j, MK_WAVE);
+      const int within = (t0 + j - t_begin) % ML_CHUNK;
+      if (within == 0) {
+        m_start = m;
+        own = -INFINITY;
+        sum = 0.f;
+      }
+      const float own_before = own;
+      m = fmaxf(b + m, a);
+      own = fmaxf(b + own, a);
+      sum += b;
+      if (lane == j) {
+        my_m = m;
+        my_own = own;
+        my_own_before = own_before;
+        my_sum = sum;
+        my_start = m_start;
+      }
+      if ((within == ML_CHUNK - 1 || t0 + j == t_end - 1) && lane == j) {
+        float* at = ends + ((size_t)(chunk + (t0 + j - t_begin) / ML_CHUNK) * heads + head) * 2;
+        at[0] = expf(sum + m_start - m);
+        at[1] = expf(own - m);
+      }
+    }
+    if (lane < count) {
+      float* at = gates + ((size_t)(t0 + lane) * heads + head) * ML_GATE_FIELDS;
+      at[0] = expf(log_keep + my_own_before - my_own);     // 0 at a chunk's first token
+      at[1] = expf(log_in - my_own);
+      at[2] = expf(my_sum + my_start - my_m);
+      at[3] = expf(my_own - my_m);
+      at[4] = expf(-my_m);
+    }
+  }
+  if (lane < copies) m_at[lane] = m;
+  for (int i = MK_WAVE + lane; i < copies; i += MK_WAVE) m_at[i] = m;
+}
+
+// MODE 0: a sequence's tokens from its slot's state, which is left for the next step.
+// MODE 1: a chunk's tokens from a zero state under the chunk's own running maximum; numerators
+//         into out, n . q into side, the chunk's last state into `chunks`.
+// MODE 2: a chunk's start state (from `chunks`) read by its queries and put together with what
+//         MODE 1 left.
+template <int R, int MODE>
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(
     const float* __restrict__ proj, int proj_stride, int q_col, int k_col, int v_col, int i_col,
     int f_col, float q_scale, float gate_cap, const int* __restrict__ cu_q,
     const int* __restrict__ slots, float* __restrict__ state, long long slot_stride, int heads,
-    int dim, int vdim, float* __restrict__ out) {
+    int dim, int vdim, float* __restrict__ out, const float* __restrict__ gates,
+    float* __restrict__ side, float* __restrict__ chunks, int num_seqs) {
   constexpr int DIM = R * 8;     // rows the lanes of a column hold between them (>= dim)
   constexpr int TOKENS = ML_TOKENS;
   __shared__ __align__(16) float q_s[TOKENS][DIM];
   __shared__ __align__(16) float k_s[TOKENS][DIM];
   __shared__ float v_s[TOKENS][ML_COLUMNS];
   __shared__ float gi_s[TOKENS], gf_s[TOKENS], keep_s[TOKENS], take_s[TOKENS], floor_s[TOKENS];
+  __shared__ float side_s[TOKENS];
   __shared__ float m_s;
-  const int seq = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * ML_COLUMNS;
+  const int head = blockIdx.y, col0 = blockIdx.z * ML_COLUMNS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int in_wave = lane & 7;
   const bool counts = in_wave == ML_WAVE_COLUMNS;       // this lane's column is n
   const int local = wave * ML_WAVE_COLUMNS + in_wave;   // among the workgroup's columns of S
   const int col = col0 + local;
   const int slice = lane >> 3, row0 = slice * R;
-  const int t_begin = cu_q[seq], t_end = cu_q[seq + 1];
+  int seq = blockIdx.x, t_begin, t_end;
+  if (MODE == 0) {
+    t_begin = cu_q[seq];
+    t_end = cu_q[seq + 1];
+  } else {
+    chunk_span(cu_q, num_seqs, blockIdx.x, seq, t_begin, t_end);
+  }
   if (t_begin >= t_end) return;
   const bool live = !counts && col < vdim;
-  float* slot = state + (size_t)slots[seq] * slot_stride;
-  float* s_at = slot + (size_t)head * dim * vdim;
-  const size_t copy = (size_t)head * gridDim.z + blockIdx.z;
-  float* n_at = slot + (size_t)heads * dim * vdim + copy * dim;
-  float* m_at = slot + (size_t)heads * dim * vdim + (size_t)heads * gridDim.z * dim + copy;
+  // MODE 0: the slot (a copy of n and m for every workgroup of the head); else the chunk's
+  // place in the workspace: [dim, vdim] of S, then [dim] of n
+  float* s_at;
+  float* n_at;
+  float* m_at = nullptr;
+  if (MODE == 0) {
+    float* slot = state + (size_t)slots[seq] * slot_stride;
+    const size_t copy = (size_t)head * gridDim.z + blockIdx.z;
+    s_at = slot + (size_t)head * dim * vdim;
+    n_at = slot + (size_t)heads * dim * vdim + copy * dim;
+    m_at = slot + (size_t)heads * dim * vdim + (size_t)heads * gridDim.z * dim + copy;
+  } else {
+    s_at = chunks + ((size_t)blockIdx.x * heads + head) * ((size_t)dim * vdim + dim);
+    n_at = s_at + (size_t)dim * vdim;
+  }
 
   float s[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int row = row0 + i;
     float got = 0.f;
-    if (row < dim) {
+    if (MODE != 1 && row < dim) {
       if (counts) got = n_at[row];
       else if (live) got = s_at[(size_t)row * vdim + col];
     }
     s[i] = got;
   }
-  float m_run = *m_at;
+  float m_run = MODE == 0 ? *m_at : 0.f;
 
   for (int t0 = t_begin; t0 < t_end; t0 += TOKENS) {
     const int count = min(TOKENS, t_end - t0);
@@ -91,52 +223,62 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
       if (row < dim) {
         const float* base = proj + (size_t)(t0 + tt) * proj_stride + head * dim + row;
         qv = base[q_col] * q_scale;
-        kv = base[k_col];
+        if (MODE != 2) kv = base[k_col];
       }
       q_s[tt][row] = qv;
-      k_s[tt][row] = kv;
+      if (MODE != 2) k_s[tt][row] = kv;
     }
+    // the values; in pass 2, in their place, what pass 1 left in out for these columns
     for (int e = tid; e < count * ML_COLUMNS; e += 256) {
       const int tt = e / ML_COLUMNS, c = e - tt * ML_COLUMNS;
-      v_s[tt][c] = col0 + c < vdim
-          ? proj[(size_t)(t0 + tt) * proj_stride + v_col + head * vdim + col0 + c] : 0.f;
-    }
-    if (tid < count) {
-      const float* row = proj + (size_t)(t0 + tid) * proj_stride;
-      float a = row[i_col + head], b = row[f_col + head];
-      if (gate_cap > 0.f) {
-        a = gate_cap * tanhf(a / gate_cap);
-        b = gate_cap * tanhf(b / gate_cap);
+      float got = 0.f;
+      if (col0 + c < vdim) {
+        got = MODE == 2 ? out[(size_t)(t0 + tt) * heads * vdim + head * vdim + col0 + c]
+                        : proj[(size_t)(t0 + tt) * proj_stride + v_col + head * vdim + col0 + c];
       }
-      gi_s[tid] = a;
-      gf_s[tid] = log_sigmoid(b);
+      v_s[tt][c] = got;
+    }
+    if (MODE == 0) {
+      if (tid < count) {
+        activated_gates(proj + (size_t)(t0 + tid) * proj_stride, i_col, f_col, head, gate_cap,
+                        gi_s[tid], gf_s[tid]);
+      }
+      __syncthreads();
+      if (tid < count) {
+        float m = m_run, before = m_run;
+        for (int j = 0; j <= tid; ++j) {
+          before = m;
+          m = fmaxf(gf_s[j] + m, gi_s[j]);
+        }
+        keep_s[tid] = expf(gf_s[tid] + before - m);
+        take_s[tid] = expf(gi_s[tid] - m);
+        floor_s[tid] = expf(-m);
+        if (tid == count - 1) m_s = m;
+      }
+    } else if (tid < count) {
+      const float* g = gates + ((size_t)(t0 + tid) * heads + head) * ML_GATE_FIELDS;
+      keep_s[tid] = MODE == 1 ? g[0] : g[2];     // pass 2: w1 and w2 in their places
+      take_s[tid] = MODE == 1 ? g[1] : g[3];
+      floor_s[tid] = g[4];
+      if (MODE == 2) side_s[tid] = side[(size_t)(t0 + tid) * heads + head];
     }
     __syncthreads();
-    if (tid < count) {
-      float m = m_run, before = m_run;
-      for (int j = 0; j <= tid; ++j) {
-        before = m;
-        m = fmaxf(gf_s[j] + m, gi_s[j]);
-      }
-      keep_s[tid] = expf(gf_s[tid] + before - m);
-      take_s[tid] = expf(gi_s[tid] - m);
-      floor_s[tid] = expf(-m);
-      if (tid == count - 1) m_s = m;
-    }
-    __syncthreads();
-    m_run = m_s;
+    if (MODE == 0) m_run = m_s;
     for (int tt = 0; tt < count; ++tt) {
       const float keep = keep_s[tt];
-      const float tv = take_s[tt] * (counts ? 1.f : v_s[tt][min(local, ML_COLUMNS - 1)]);
+      const float held = counts ? 1.f : v_s[tt][min(local, ML_COLUMNS - 1)];
+      const float tv = take_s[tt] * held;
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < R; i += 4) {
         const float4 q4 = *(const float4*)&q_s[tt][row0 + i];
-        const float4 k4 = *(const float4*)&k_s[tt][row0 + i];
-        s[i] = fmaf(k4.x, tv, keep * s[i]);
-        s[i + 1] = fmaf(k4.y, tv, keep * s[i + 1]);
-        s[i + 2] = fmaf(k4.z, tv, keep * s[i + 2]);
-        s[i + 3] = fmaf(k4.w, tv, keep * s[i + 3]);
+        if (MODE != 2) {
+          const float4 k4 = *(const float4*)&k_s[tt][row0 + i];
+          s[i] = fmaf(k4.x, tv, keep * s[i]);
+          s[i + 1] = fmaf(k4.y, tv, keep * s[i + 1]);
+          s[i + 2] = fmaf(k4.z, tv, keep * s[i + 2]);
+          s[i + 3] = fmaf(k4.w, tv, keep * s[i + 3]);
+        }
         o = fmaf(s[i], q4.x, o);
         o = fmaf(s[i + 1], q4.y, o);
         o = fmaf(s[i + 2], q4.z, o);
@@ -145,15 +287,24 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
       o += __shfl_xor(o, 8, MK_WAVE);
       o += __shfl_xor(o, 16, MK_WAVE);
       o += __shfl_xor(o, 32, MK_WAVE);
-      const float nq = __shfl(o, lane | 7, MK_WAVE);
-      if (slice == 0 && live) {
-        out[(size_t)(t0 + tt) * heads * vdim + head * vdim + col] =
-            o / (fmaxf(fabsf(nq), floor_s[tt]) + 1e-6f);
+      float nq = __shfl(o, lane | 7, MK_WAVE);
+      float* at = out + (size_t)(t0 + tt) * heads * vdim + head * vdim + col;
+      if (MODE == 1) {
+        if (slice == 0 && live) *at = o;
+        if (blockIdx.z == 0 && tid == ML_WAVE_COLUMNS) side[(size_t)(t0 + tt) * heads + head] = nq;
+        continue;
       }
+      if (MODE == 2) {      // keep = w1, take = w2, held = pass 1's numerator
+        o = fmaf(keep, o, tv);
+        nq = fmaf(keep, nq, take_s[tt] * side_s[tt]);
+      }
+      if (slice == 0 && live) *at = o / (fmaxf(fabsf(nq), floor_s[tt]) + 1e-6f);
     }
   }
-  // S by the lanes that own its columns; the workgroup's n by its first wavefront
-  const bool keeps_n = counts && wave == 0;
+  if (MODE == 2) return;
+  // S by the lanes that own its columns; n by the first wavefront (MODE 0: of every workgroup,
+  // into its own copy; MODE 1: of the head's first workgroup)
+  const bool keeps_n = counts && wave == 0 && (MODE == 0 || blockIdx.z == 0);
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int row = row0 + i;
@@ -161,7 +312,54 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
     if (live) s_at[(size_t)row * vdim + col] = s[i];
     else if (keeps_n) n_at[row] = s[i];
   }
-  if (tid == 0) *m_at = m_run;
+  if (MODE == 0 && tid == 0) *m_at = m_run;
+}
+
+// The chunks' start states, one sequence's after the other: a thread owns one entry of a
+// head's S or n, takes it from the slot, leaves in every chunk's place what the chunk starts
+// from, and puts what the last chunk ends with back into the slot (n into every copy).
+__global__ __launch_bounds__(256) void mlstm_carry_kernel(
+    const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ state,
+    long long slot_stride, const float* __restrict__ ends, float* __restrict__ chunks, int heads,
+    int dim, int vdim, int copies) {
+  const int seq = blockIdx.x, head = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
+  const int entries = dim * vdim + dim;
+  if (e >= entries) return;
+  int first = 0;
+  for (int i = 0; i < seq; ++i) first += (cu_q[i + 1] - cu_q[i] + ML_CHUNK - 1) / ML_CHUNK;
+  const int tokens = cu_q[seq + 1] - cu_q[seq];
+  if (tokens <= 0) return;
+  float* slot = state + (size_t)slots[seq] * slot_stride;
+  const bool of_n = e >= dim * vdim;
+  float* mine = of_n ? slot + (size_t)heads * dim * vdim + (size_t)head * copies * dim + (e - dim * vdim)
+                     : slot + (size_t)head * dim * vdim + e;
+  float* at = chunks + ((size_t)first * heads + head) * entries + e;
+  const float* w = ends + ((size_t)first * heads + head) * 2;
+  const size_t step = (size_t)heads * entries;
+  const int count = (tokens + ML_CHUNK - 1) / ML_CHUNK;
+  float s = *mine;
+  // eight chunks' ends are asked for at a time, so that their ways to memory overlap
+  for (int c0 = 0; c0 < count; c0 += 8) {
+    float ended[8], w1[8], w2[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool there = c0 + j < count;
+      ended[j] = there ? at[(size_t)(c0 + j) * step] : 0.f;
+      w1[j] = there ? w[(size_t)(c0 + j) * heads * 2] : 0.f;
+      w2[j] = there ? w[(size_t)(c0 + j) * heads * 2 + 1] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (c0 + j >= count) break;
+      at[(size_t)(c0 + j) * step] = s;
+      s = fmaf(w1[j], s, w2[j] * ended[j]);
+    }
+  }
+  if (of_n) {
+    for (int c = 0; c < copies; ++c) mine[(size_t)c * dim] = s;
+  } else {
+    *mine = s;
+  }
 }
 
 }  // namespace
@@ -172,11 +370,21 @@ extern "C" long long mk_mlstm_state_floats(int heads, int dim, int vdim) {
   return (long long)heads * ((long long)dim * vdim + copies * (dim + 1));
 }
 
+extern "C" int mk_mlstm_chunk_tokens(void) { return ML_CHUNK; }
+
+extern "C" long long mk_mlstm_scan_workspace(int total_chunks, int tokens, int heads, int dim,
+                                             int vdim) {
+  if (total_chunks < 0 || tokens < 0 || heads <= 0 || dim <= 0 || vdim <= 0) return -1;
+  // the chunks' states, their end weights, the tokens' gates and n . q
+  return (long long)total_chunks * heads * ((long long)dim * vdim + dim + 2) +
+         (long long)tokens * heads * (ML_GATE_FIELDS + 1);
+}
+
 extern "C" int mk_mlstm_scan(const float* proj, int proj_stride, int q_col, int k_col, int v_col,
                              int i_col, int f_col, float q_scale, float gate_cap, const int* cu_q,
                              const int* slots, float* state, long long slot_stride, int heads,
                              int dim, int vdim, float* out, int tokens, int num_seqs,
-                             hipStream_t stream) {
+                             int total_chunks, float* workspace, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && num_seqs >= 0 && heads > 0 && dim > 0 && vdim > 0, "mlstm: bad sizes");
   MK_REQUIRE(dim <= ML_MAX_DIM, "mlstm: heads of %d dims exceed the supported %d", dim, ML_MAX_DIM);
   MK_REQUIRE(slot_stride >= mk_mlstm_state_floats(heads, dim, vdim),
@@ -191,16 +399,42 @@ extern "C" int mk_mlstm_scan(const float* proj, int proj_stride, int q_col, int 
   MK_REQUIRE(heads <= 65535 && columns <= 65535, "mlstm: too many heads or columns");
   if (tokens == 0 || num_seqs == 0) return 0;
   MK_REQUIRE(proj && cu_q && slots && state && out, "mlstm: null operand");
+  MK_REQUIRE(total_chunks >= 0 && (total_chunks == 0 || workspace),
+             "mlstm: chunks without a workspace");
   const int per_lane = (dim + 7) / 8;
-#define ML_LAUNCH(R)                                                                           \
-  mlstm_scan_kernel<R><<<dim3(num_seqs, heads, columns), 256, 0, stream>>>(                    \
-      proj, proj_stride, q_col, k_col, v_col, i_col, f_col, q_scale, gate_cap, cu_q, slots,    \
-      state, slot_stride, heads, dim, vdim, out)
-  if (per_lane <= 4) ML_LAUNCH(4);
-  else if (per_lane <= 8) ML_LAUNCH(8);
-  else if (per_lane <= 16) ML_LAUNCH(16);
-  else ML_LAUNCH(32);
+  float* chunk_states = workspace;
+  float* ends = workspace ? chunk_states + (size_t)total_chunks * heads * ((size_t)dim * vdim + dim) : nullptr;
+  float* gates = workspace ? ends + (size_t)total_chunks * heads * 2 : nullptr;
+  float* side = workspace ? gates + (size_t)tokens * heads * ML_GATE_FIELDS : nullptr;
+#define ML_LAUNCH_R(R, MODE, first)                                                             \
+  mlstm_scan_kernel<R, MODE><<<dim3(first, heads, columns), 256, 0, stream>>>(                  \
+      proj, proj_stride, q_col, k_col, v_col, i_col, f_col, q_scale, gate_cap, cu_q, slots,     \
+      state, slot_stride, heads, dim, vdim, out, gates, side, chunk_states, num_seqs)
+#define ML_LAUNCH(MODE, first)                                                                  \
+  do {                                                                                          \
+    if (per_lane <= 4) ML_LAUNCH_R(4, MODE, first);                                             \
+    else if (per_lane <= 8) ML_LAUNCH_R(8, MODE, first);                                        \
+    else if (per_lane <= 16) ML_LAUNCH_R(16, MODE, first);                                      \
+    else ML_LAUNCH_R(32, MODE, first);                                                          \
+  } while (0)
+  if (total_chunks == 0) {
+    ML_LAUNCH(0, num_seqs);
+    MK_LAUNCH_CHECK("mlstm_scan");
+    return 0;
+  }
+  mlstm_gates_kernel<<<dim3(num_seqs, heads), MK_WAVE, 0, stream>>>(
+      proj, proj_stride, i_col, f_col, gate_cap, cu_q, slots, state, slot_stride, heads, dim, vdim,
+      columns, gates, ends);
+  MK_LAUNCH_CHECK("mlstm_gates");
+  ML_LAUNCH(1, total_chunks);
+  MK_LAUNCH_CHECK("mlstm_scan (chunks)");
+  const int entries = dim * vdim + dim;
+  mlstm_carry_kernel<<<dim3(num_seqs, heads, (entries + 255) / 256), 256, 0, stream>>>(
+      cu_q, slots, state, slot_stride, ends, chunk_states, heads, dim, vdim, columns);
+  MK_LAUNCH_CHECK("mlstm_carry");
+  ML_LAUNCH(2, total_chunks);
 #undef ML_LAUNCH
-  MK_LAUNCH_CHECK("mlstm_scan");
+#undef ML_LAUNCH_R
+  MK_LAUNCH_CHECK("mlstm_scan (start states)");
   return 0;
 }

@@ -555,13 +555,29 @@ void mlstm(Launch& l, const void* x, int m, int hidden, const MlstmArgs& a,
                                            nullptr, kF32, false);
   float* y = (float*)l.alloc((size_t)m * inner * 4);
   void* normed = l.alloc((size_t)m * inner * l.elem());
+  // a step with a sequence longer than a chunk runs the recurrence in chunks side by side
+  const KernelTable& core = need_core();
+  const int chunk = core.mk_mlstm_chunk_tokens();
+  int total_chunks = 0, longest = 0;
+  for (int i = 0; i < step.num_seqs; ++i) {
+    total_chunks += (step.counts[i] + chunk - 1) / chunk;
+    longest = std::max(longest, step.counts[i]);
+  }
+  if (longest <= chunk) total_chunks = 0;
+  float* scan_ws = nullptr;
+  if (total_chunks) {
+    const long long floats = core.mk_mlstm_scan_workspace(total_chunks, m, a.heads, a.dim, a.vdim);
+    if (floats < 0) throw KernelError("mlstm: the recurrence does not run these sizes");
+    scan_ws = (float*)l.alloc((size_t)floats * 4);
+  }
   if (!l.dry() && m > 0) {
     const KernelTable& t = need_core();
     if (!a.state) throw KernelError("mlstm: no state tensor");
     const int gates = 2 * qk + 2 * inner;
     check_core(t.mk_mlstm_scan(proj, width, 0, qk, 2 * qk, gates, gates + a.heads, a.q_scale,
                                a.gate_cap, step.cu_q, step.state_slots, a.state, a.slot_floats,
-                               a.heads, a.dim, a.vdim, y, m, step.num_seqs, l.stream()),
+                               a.heads, a.dim, a.vdim, y, m, step.num_seqs, total_chunks, scan_ws,
+                               l.stream()),
                "mlstm_scan");
     check_core(t.mk_head_norm_gate(y, normed, l.dtype(), proj + 2 * qk + inner, width, a.eps, m,
                                    a.heads, a.vdim, a.norm, MK_GATE_SIGMOID, l.stream()),

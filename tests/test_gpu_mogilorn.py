@@ -213,16 +213,17 @@ def test_the_memory_s_state_size_is_the_kernel_library_s():
 
 @pytest.mark.parametrize("dtype", BOTH)
 def test_matrix_memory_long_portions_and_long_decoding(dtype):
-    """A portion of 300 tokens, odd cuts, then 200 tokens one by one, gates that let the
-    running maximum rise and fall."""
+    """Portions of 300, 1, 129, 128 and 2 tokens (more than 128 tokens of a sequence run in
+    chunks side by side whose start states are carried), then 200 tokens one by one, gates that
+    let the running maximum rise and fall."""
     hidden, m = 64, memory(2, 16, 40, gate_cap=9.0)
     part = matrix_memory(hidden, m)
     params = bind_random(part, dtype, scale=0.2, seed=21)
     rebind(part, params, dtype, slow_and_loud)
-    total = 540
+    total = 760
     x = rnd(total, hidden, seed=7).to(dtype).float()
-    cuts = [(0, 300), (300, 1), (301, 17), (318, 2), (320, 20)] + [(340 + i, 1) for i in range(200)]
-    got = run_mixer_in_portions(part, x.to(dtype), dtype, hidden, pages=40, portions=cuts)
+    cuts = [(0, 300), (300, 1), (301, 129), (430, 128), (558, 2)] + [(560 + i, 1) for i in range(200)]
+    got = run_mixer_in_portions(part, x.to(dtype), dtype, hidden, pages=50, portions=cuts)
 
     def run(to, r):
         w = {n: to(t) for n, t in plain_names(params).items()}
