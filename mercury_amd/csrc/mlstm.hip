@@ -24,18 +24,21 @@
 // A step with a sequence longer than ML_CHUNK tokens runs in chunks side by side.  With
 // b_j the sum of the log forget gates from the chunk's first token to its j-th, m the running
 // maximum of the whole sequence and m' the one of the chunk alone (from minus infinity):
-//   gates     one wavefront a (sequence, head) walks the gates in order and leaves, per token,
-//             the chunk's own recurrence weights exp(f_j + m'_(j-1) - m'_j), exp(i_j - m'_j),
-//             the weights w1 = exp(b_j + m_start - m_j), w2 = exp(m'_j - m_j) that put the
-//             chunk's start state and its own part together, and exp(-m_j); per chunk the
-//             same two weights at its last token; and the slot's new m;
+//   gates     one wavefront a (chunk, head): b_j and m'_j = b_j + max_(s<=j)(i_s - b_s) of the
+//             chunk's tokens by prefix sums and maxima, and with them the chunk's own
+//             recurrence weights exp(f_j + m'_(j-1) - m'_j), exp(i_j - m'_j);
 //   pass 1    every chunk's recurrence from a zero state under m' (its numerators and n . q
 //             into `out` and a side buffer, its last state into the workspace);
-//   carry     the chunks' start states one after the other,
-//             S_start(c + 1) = w1_end(c) S_start(c) + w2_end(c) S_own(c), the last into the slot;
-//   pass 2    S_start^T q_j of every token, and w1 (that) + w2 (pass 1's) over the floored
+//   carry     the chunks' start states one after the other, with the running maximum at
+//             every chunk's start, m_start(c + 1) = max(m_start(c) + b_end(c), m'_end(c)):
+//             S_start(c + 1) = exp(b_end + m_start - m_end) S_start(c) + exp(m'_end - m_end) S_own(c),
+//             the last into the slot with the last m;
+//   pass 2    S_start^T q_j of every token, and, with m_j = max(m_start + b_j, m'_j),
+//             exp(b_j + m_start - m_j) (that) + exp(m'_j - m_j) (pass 1's) over the floored
 //             denominator.
-// Every exponent above is at most zero: m_j >= b_j + m_start and m_j >= m'_j.
+// Every exponent above is at most zero (to rounding): m_j >= b_j + m_start and m_j >= m'_j.  The
+// running maximum only keeps the exponentials in range; made by prefix sums instead of step by
+// step it differs in its last bits, which reach the result through the 1e-6 alone.
 //
 // A slot holds [heads, dim, vdim] floats of S, then n [heads, B, dim] and m [heads, B] once for
 // each of the B = ceil(vdim / 28) workgroups of a head: a workgroup reads and writes a copy of
@@ -49,7 +52,8 @@
 #define ML_COLUMNS 28      // columns of a head per workgroup
 #define ML_MAX_DIM 256
 #define ML_CHUNK 128       // tokens of a chunk when a step runs in chunks
-#define ML_GATE_FIELDS 5   // per (token, head): keep', take', w1, w2, exp(-m)
+#define ML_GATE_FIELDS 4   // per (token, head): keep', take', b, m'
+#define ML_CHUNK_FIELDS 4  // per (chunk, head): b_end, m'_end, m_start, the slot's m (a sequence's first chunk)
 
 namespace {
 
@@ -87,66 +91,69 @@ __device__ __forceinline__ void chunk_span(const int* __restrict__ cu_q, int num
   t_end = min(cu_q[seq + 1], t_begin + ML_CHUNK);
 }
 
-// One wavefront a (sequence, head): the gates of the sequence's tokens in order.
-// gates [tokens, heads, ML_GATE_FIELDS]; ends [chunks, heads, 2] (w1 and w2 at a chunk's last
-// token); the slot's copies of m are read (the first) and written (all).
+__device__ __forceinline__ float wave_prefix_sum(float v, int lane) {
+#pragma unroll
+  for (int d = 1; d < MK_WAVE; d <<= 1) {
+    const float up = __shfl_up(v, d, MK_WAVE);
+    if (lane >= d) v += up;
+  }
+  return v;
+}
+
+__device__ __forceinline__ float wave_prefix_max(float v, int lane) {
+#pragma unroll
+  for (int d = 1; d < MK_WAVE; d <<= 1) {
+    const float up = __shfl_up(v, d, MK_WAVE);
+    if (lane >= d) v = fmaxf(v, up);
+  }
+  return v;
+}
+
+// One wavefront a (chunk, head): gates [tokens, heads, ML_GATE_FIELDS], ends
+// [chunks, heads, ML_CHUNK_FIELDS].
 __global__ __launch_bounds__(64) void mlstm_gates_kernel(
     const float* __restrict__ proj, int proj_stride, int i_col, int f_col, float gate_cap,
-    const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ state,
+    const int* __restrict__ cu_q, const int* __restrict__ slots, const float* __restrict__ state,
     long long slot_stride, int heads, int dim, int vdim, int copies, float* __restrict__ gates,
-    float* __restrict__ ends) {
-  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int t_begin = cu_q[seq], t_end = cu_q[seq + 1];
+    float* __restrict__ ends, int num_seqs) {
+  const int head = blockIdx.y, lane = threadIdx.x;
+  int seq, t_begin, t_end;
+  chunk_span(cu_q, num_seqs, blockIdx.x, seq, t_begin, t_end);
   if (t_begin >= t_end) return;
-  int chunk = 0;     // the sequence's first chunk among the step's
-  for (int i = 0; i < seq; ++i) chunk += (cu_q[i + 1] - cu_q[i] + ML_CHUNK - 1) / ML_CHUNK;
-  float* m_at = state + (size_t)slots[seq] * slot_stride + (size_t)heads * dim * vdim +
-                (size_t)heads * copies * dim + (size_t)head * copies;
-  float m = *m_at, own = -INFINITY, sum = 0.f, m_start = m;
+  float sum_before = 0.f, top_before = -INFINITY, own_last = -INFINITY;
   for (int t0 = t_begin; t0 < t_end; t0 += MK_WAVE) {
-    const int count = min(MK_WAVE, t_end - t0);
-    float log_in = 0.f, log_keep = 0.f;
-    if (lane < count) {
+    const bool there = t0 + lane < t_end;
+    float log_in = -INFINITY, log_keep = 0.f;
+    if (there) {
       activated_gates(proj + (size_t)(t0 + lane) * proj_stride, i_col, f_col, head, gate_cap,
                       log_in, log_keep);
     }
-    float my_m = 0.f, my_own = 0.f, my_own_before = 0.f, my_sum = 0.f, my_start = 0.f;
-    for (int j = 0; j < count; ++j) {
-      const float a = __shfl(log_in, j, MK_WAVE), b = __shfl(log_keep, j, MK_WAVE);
-      const int within = (t0 + j - t_begin) % ML_CHUNK;
-      if (within == 0) {
-        m_start = m;
-        own = -INFINITY;
-        sum = 0.f;
-      }
-      const float own_before = own;
-      m = fmaxf(b + m, a);
-      own = fmaxf(b + own, a);
-      sum += b;
-      if (lane == j) {
-        my_m = m;
-        my_own = own;
-        my_own_before = own_before;
-        my_sum = sum;
-        my_start = m_start;
-      }
-      if ((within == ML_CHUNK - 1 || t0 + j == t_end - 1) && lane == j) {
-        float* at = ends + ((size_t)(chunk + (t0 + j - t_begin) / ML_CHUNK) * heads + head) * 2;
-        at[0] = expf(sum + m_start - m);
-        at[1] = expf(own - m);
-      }
-    }
-    if (lane < count) {
+    const float sum = sum_before + wave_prefix_sum(log_keep, lane);
+    const float top = fmaxf(top_before, wave_prefix_max(log_in - sum, lane));
+    const float own = sum + top;
+    float own_before = __shfl_up(own, 1, MK_WAVE);
+    if (lane == 0) own_before = own_last;
+    if (there) {
       float* at = gates + ((size_t)(t0 + lane) * heads + head) * ML_GATE_FIELDS;
-      at[0] = expf(log_keep + my_own_before - my_own);     // 0 at a chunk's first token
-      at[1] = expf(log_in - my_own);
-      at[2] = expf(my_sum + my_start - my_m);
-      at[3] = expf(my_own - my_m);
-      at[4] = expf(-my_m);
+      at[0] = expf(fminf(log_keep + own_before - own, 0.f));     // 0 at a chunk's first token
+      at[1] = expf(log_in - own);
+      at[2] = sum;
+      at[3] = own;
+    }
+    const int last = min(MK_WAVE, t_end - t0) - 1;
+    sum_before = __shfl(sum, last, MK_WAVE);
+    top_before = __shfl(top, last, MK_WAVE);
+    own_last = __shfl(own, last, MK_WAVE);
+  }
+  if (lane == 0) {
+    float* at = ends + ((size_t)blockIdx.x * heads + head) * ML_CHUNK_FIELDS;
+    at[0] = sum_before;
+    at[1] = own_last;
+    if (t_begin == cu_q[seq]) {     // the sequence's first chunk keeps the m the slot holds
+      at[3] = state[(size_t)slots[seq] * slot_stride + (size_t)heads * dim * vdim +
+                    (size_t)heads * copies * dim + (size_t)head * copies];
     }
   }
-  if (lane < copies) m_at[lane] = m;
-  for (int i = MK_WAVE + lane; i < copies; i += MK_WAVE) m_at[i] = m;
 }
 
 // MODE 0: a sequence's tokens from its slot's state, which is left for the next step.
@@ -160,7 +167,8 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
     int f_col, float q_scale, float gate_cap, const int* __restrict__ cu_q,
     const int* __restrict__ slots, float* __restrict__ state, long long slot_stride, int heads,
     int dim, int vdim, float* __restrict__ out, const float* __restrict__ gates,
-    float* __restrict__ side, float* __restrict__ chunks, int num_seqs) {
+    float* __restrict__ side, float* __restrict__ chunks, const float* __restrict__ ends,
+    int num_seqs) {
   constexpr int DIM = R * 8;     // rows the lanes of a column hold between them (>= dim)
   constexpr int TOKENS = ML_TOKENS;
   __shared__ __align__(16) float q_s[TOKENS][DIM];
@@ -257,10 +265,17 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
       }
     } else if (tid < count) {
       const float* g = gates + ((size_t)(t0 + tid) * heads + head) * ML_GATE_FIELDS;
-      keep_s[tid] = MODE == 1 ? g[0] : g[2];     // pass 2: w1 and w2 in their places
-      take_s[tid] = MODE == 1 ? g[1] : g[3];
-      floor_s[tid] = g[4];
-      if (MODE == 2) side_s[tid] = side[(size_t)(t0 + tid) * heads + head];
+      if (MODE == 1) {
+        keep_s[tid] = g[0];
+        take_s[tid] = g[1];
+      } else {     // pass 2: the weights of the start state and of the chunk's own part
+        const float m_start = ends[((size_t)blockIdx.x * heads + head) * ML_CHUNK_FIELDS + 2];
+        const float m = fmaxf(m_start + g[2], g[3]);
+        keep_s[tid] = expf(fminf(g[2] + m_start - m, 0.f));
+        take_s[tid] = expf(fminf(g[3] - m, 0.f));
+        floor_s[tid] = expf(-m);
+        side_s[tid] = side[(size_t)(t0 + tid) * heads + head];
+      }
     }
     __syncthreads();
     if (MODE == 0) m_run = m_s;
@@ -317,10 +332,12 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
 
 // The chunks' start states, one sequence's after the other: a thread owns one entry of a
 // head's S or n, takes it from the slot, leaves in every chunk's place what the chunk starts
-// from, and puts what the last chunk ends with back into the slot (n into every copy).
+// from, and puts what the last chunk ends with back into the slot (n into every copy).  Every
+// thread walks the running maximum along; the head's first thread leaves it at every chunk's
+// start for pass 2 and puts the last one into the slot's copies.
 __global__ __launch_bounds__(256) void mlstm_carry_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ state,
-    long long slot_stride, const float* __restrict__ ends, float* __restrict__ chunks, int heads,
+    long long slot_stride, float* __restrict__ ends, float* __restrict__ chunks, int heads,
     int dim, int vdim, int copies) {
   const int seq = blockIdx.x, head = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
   const int entries = dim * vdim + dim;
@@ -334,31 +351,39 @@ __global__ __launch_bounds__(256) void mlstm_carry_kernel(
   float* mine = of_n ? slot + (size_t)heads * dim * vdim + (size_t)head * copies * dim + (e - dim * vdim)
                      : slot + (size_t)head * dim * vdim + e;
   float* at = chunks + ((size_t)first * heads + head) * entries + e;
-  const float* w = ends + ((size_t)first * heads + head) * 2;
-  const size_t step = (size_t)heads * entries;
+  float* w = ends + ((size_t)first * heads + head) * ML_CHUNK_FIELDS;
+  const size_t step = (size_t)heads * entries, w_step = (size_t)heads * ML_CHUNK_FIELDS;
   const int count = (tokens + ML_CHUNK - 1) / ML_CHUNK;
   float s = *mine;
+  float m = w[3];
   // eight chunks' ends are asked for at a time, so that their ways to memory overlap
   for (int c0 = 0; c0 < count; c0 += 8) {
-    float ended[8], w1[8], w2[8];
+    float ended[8], sum[8], own[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const bool there = c0 + j < count;
       ended[j] = there ? at[(size_t)(c0 + j) * step] : 0.f;
-      w1[j] = there ? w[(size_t)(c0 + j) * heads * 2] : 0.f;
-      w2[j] = there ? w[(size_t)(c0 + j) * heads * 2 + 1] : 0.f;
+      sum[j] = there ? w[(size_t)(c0 + j) * w_step] : 0.f;
+      own[j] = there ? w[(size_t)(c0 + j) * w_step + 1] : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if (c0 + j >= count) break;
       at[(size_t)(c0 + j) * step] = s;
-      s = fmaf(w1[j], s, w2[j] * ended[j]);
+      if (e == 0) w[(size_t)(c0 + j) * w_step + 2] = m;
+      const float m_end = fmaxf(m + sum[j], own[j]);
+      s = fmaf(expf(fminf(sum[j] + m - m_end, 0.f)), s, expf(fminf(own[j] - m_end, 0.f)) * ended[j]);
+      m = m_end;
     }
   }
   if (of_n) {
     for (int c = 0; c < copies; ++c) mine[(size_t)c * dim] = s;
   } else {
     *mine = s;
+  }
+  if (e == 0) {
+    float* m_at = slot + (size_t)heads * dim * vdim + (size_t)heads * copies * dim + (size_t)head * copies;
+    for (int c = 0; c < copies; ++c) m_at[c] = m;
   }
 }
 
@@ -375,8 +400,8 @@ extern "C" int mk_mlstm_chunk_tokens(void) { return ML_CHUNK; }
 extern "C" long long mk_mlstm_scan_workspace(int total_chunks, int tokens, int heads, int dim,
                                              int vdim) {
   if (total_chunks < 0 || tokens < 0 || heads <= 0 || dim <= 0 || vdim <= 0) return -1;
-  // the chunks' states, their end weights, the tokens' gates and n . q
-  return (long long)total_chunks * heads * ((long long)dim * vdim + dim + 2) +
+  // the chunks' states and scalars, the tokens' gates and n . q
+  return (long long)total_chunks * heads * ((long long)dim * vdim + dim + ML_CHUNK_FIELDS) +
          (long long)tokens * heads * (ML_GATE_FIELDS + 1);
 }
 
@@ -404,12 +429,12 @@ extern "C" int mk_mlstm_scan(const float* proj, int proj_stride, int q_col, int 
   const int per_lane = (dim + 7) / 8;
   float* chunk_states = workspace;
   float* ends = workspace ? chunk_states + (size_t)total_chunks * heads * ((size_t)dim * vdim + dim) : nullptr;
-  float* gates = workspace ? ends + (size_t)total_chunks * heads * 2 : nullptr;
+  float* gates = workspace ? ends + (size_t)total_chunks * heads * ML_CHUNK_FIELDS : nullptr;
   float* side = workspace ? gates + (size_t)tokens * heads * ML_GATE_FIELDS : nullptr;
 #define ML_LAUNCH_R(R, MODE, first)                                                             \
   mlstm_scan_kernel<R, MODE><<<dim3(first, heads, columns), 256, 0, stream>>>(                  \
       proj, proj_stride, q_col, k_col, v_col, i_col, f_col, q_scale, gate_cap, cu_q, slots,     \
-      state, slot_stride, heads, dim, vdim, out, gates, side, chunk_states, num_seqs)
+      state, slot_stride, heads, dim, vdim, out, gates, side, chunk_states, ends, num_seqs)
 #define ML_LAUNCH(MODE, first)                                                                  \
   do {                                                                                          \
     if (per_lane <= 4) ML_LAUNCH_R(4, MODE, first);                                             \
@@ -422,9 +447,9 @@ extern "C" int mk_mlstm_scan(const float* proj, int proj_stride, int q_col, int 
     MK_LAUNCH_CHECK("mlstm_scan");
     return 0;
   }
-  mlstm_gates_kernel<<<dim3(num_seqs, heads), MK_WAVE, 0, stream>>>(
+  mlstm_gates_kernel<<<dim3(total_chunks, heads), MK_WAVE, 0, stream>>>(
       proj, proj_stride, i_col, f_col, gate_cap, cu_q, slots, state, slot_stride, heads, dim, vdim,
-      columns, gates, ends);
+      columns, gates, ends, num_seqs);
   MK_LAUNCH_CHECK("mlstm_gates");
   ML_LAUNCH(1, total_chunks);
   MK_LAUNCH_CHECK("mlstm_scan (chunks)");
