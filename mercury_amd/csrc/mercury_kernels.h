@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 37
+#define MK_ABI_VERSION 38
 
 // Gate activations of a gated feed-forward: SILU is silu(g) * u; SWISH_CLAMP is
 // g' * sigmoid(alpha * g') * (u' + beta) with g' = min(g, limit), u' = clamp(u, -limit, limit);
@@ -258,10 +258,12 @@ int mk_normed_sum(float* h, const float* ya, const float* pa, int na, const void
 
 // h[t, :] += scale .* (rmsnorm(y[t, :] + its `count` partial sums p[k * stride + .]) * weight):
 // a sublayer's output normed before it enters the stream, times a stored vector per channel
-// (`scale`, float32 or null).
+// (`scale`, float32 or null).  x_out (or null): the new h once more, in x_dtype, for a sublayer
+// that reads the stream itself.
 int mk_norm_scale_add(float* h, const float* y, const float* partials, int count,
                       long long stride, const void* weight, int weight_dtype, const float* scale,
-                      float eps, int tokens, int hidden, hipStream_t stream);
+                      float eps, int tokens, int hidden, void* x_out, int x_dtype,
+                      hipStream_t stream);
 
 // Differential attention's tail.  a [T, heads, 2, dv] (`dtype`) holds two maps' outputs per
 // head; o = a1 - lambda * a2 is divided by its root mean square over dv (eps inside the root),

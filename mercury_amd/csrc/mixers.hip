@@ -11,7 +11,8 @@
 //   mk_stream_cast     the residual stream itself as a sublayer's input;
 //   mk_normed_sum      h += mult * (rmsnorm(a) * wa + rmsnorm(b) * wb): mixers side by side;
 //   mk_norm_scale_add  h += scale .* (rmsnorm(y) * w): a sublayer's output normed before it
-//                      enters the stream, times a stored vector per channel;
+//                      enters the stream, times a stored vector per channel; the new stream
+//                      may go out once more in the compute dtype, for a sublayer that reads it;
 //   mk_diff_heads      two attention maps per head combined, normed per head and gated;
 //   mk_concat_cast     [a | b] row by row, in the compute dtype (the operand of a projection
 //                      of two streams);
@@ -195,11 +196,11 @@ __global__ __launch_bounds__(256) void normed_sum_kernel(
 
 // One workgroup per token (or several that share its outputs, each making the sum of squares
 // for itself in the same order).
-template <typename TW>
+template <typename TW, typename TX>
 __global__ __launch_bounds__(256) void norm_scale_add_kernel(
     float* __restrict__ h, const float* __restrict__ y, const float* __restrict__ partials,
     int count, size_t stride, const void* __restrict__ weight, const float* __restrict__ scale,
-    float eps, int hidden) {
+    float eps, int hidden, TX* __restrict__ x_out) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * hidden;
   auto value = [&](int i) {
@@ -215,7 +216,9 @@ __global__ __launch_bounds__(256) void norm_scale_add_kernel(
   const float r = rsqrtf(block_sum(sq, scratch) / (float)hidden + eps);
   for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < hidden; i += gridDim.y * blockDim.x) {
     const float normed = value(i) * r * weight_at<TW>(weight, i);
-    h[base + i] += scale ? scale[i] * normed : normed;
+    const float sum = h[base + i] + (scale ? scale[i] * normed : normed);
+    h[base + i] = sum;
+    if (x_out) Elem<TX>::store(x_out + base + i, sum);
   }
 }
 
@@ -223,11 +226,11 @@ __global__ __launch_bounds__(256) void norm_scale_add_kernel(
 // entries in registers between the sum of squares and the output, and the partial sums of an
 // entry are read side by side (in the same order of addition).
 #define NSA_NV 16
-template <typename TW, int NV>
+template <typename TW, int NV, typename TX>
 __global__ __launch_bounds__(256) void norm_scale_add_held_kernel(
     float* __restrict__ h, const float* __restrict__ y, const float* __restrict__ partials,
     int count, size_t stride, const void* __restrict__ weight, const float* __restrict__ scale,
-    float eps, int hidden) {
+    float eps, int hidden, TX* __restrict__ x_out) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * hidden;
   float vals[NV];
@@ -265,7 +268,9 @@ __global__ __launch_bounds__(256) void norm_scale_add_held_kernel(
     const int i = threadIdx.x + j * 256;
     if (i < hidden) {
       const float normed = vals[j] * r * weight_at<TW>(weight, i);
-      h[base + i] += scale ? scale[i] * normed : normed;
+      const float sum = h[base + i] + (scale ? scale[i] * normed : normed);
+      h[base + i] = sum;
+      if (x_out) Elem<TX>::store(x_out + base + i, sum);
     }
   }
 }
@@ -436,17 +441,25 @@ extern "C" int mk_normed_sum(float* h, const float* ya, const float* pa, int na,
 extern "C" int mk_norm_scale_add(float* h, const float* y, const float* partials, int count,
                                  long long stride, const void* weight, int weight_dtype,
                                  const float* scale, float eps, int tokens, int hidden,
-                                 hipStream_t stream) {
+                                 void* x_out, int x_dtype, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && hidden > 0, "norm_scale_add: bad sizes");
+  MK_REQUIRE(!x_out || x_dtype == MK_F32 || x_dtype == MK_BF16, "norm_scale_add: x dtype %d", x_dtype);
+  const bool x_bf16 = x_out && x_dtype == MK_BF16;
   MK_REQUIRE(count >= 0 && (count == 0 || partials), "norm_scale_add: partial sums without a buffer");
   MK_REQUIRE((y || count) && weight && h, "norm_scale_add: no operand");
   MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "norm_scale_add: weight dtype %d",
              weight_dtype);
   if (tokens == 0) return 0;
   if (hidden <= 256 * NSA_NV) {
-#define NSA_LAUNCH(TW, NV)                                        \
-  norm_scale_add_held_kernel<TW, NV><<<tokens, 256, 0, stream>>>( \
-      h, y, partials, count, (size_t)stride, weight, scale, eps, hidden)
+#define NSA_LAUNCH(TW, NV)                                                                  \
+  do {                                                                                      \
+    if (x_bf16)                                                                             \
+      norm_scale_add_held_kernel<TW, NV, bf16_t><<<tokens, 256, 0, stream>>>(               \
+          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden, (bf16_t*)x_out); \
+    else                                                                                    \
+      norm_scale_add_held_kernel<TW, NV, float><<<tokens, 256, 0, stream>>>(                \
+          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden, (float*)x_out); \
+  } while (0)
     if (weight_dtype == MK_F32) {
       if (hidden <= 256 * 4) NSA_LAUNCH(float, 4);
       else if (hidden <= 256 * 8) NSA_LAUNCH(float, 8);
@@ -461,12 +474,18 @@ extern "C" int mk_norm_scale_add(float* h, const float* y, const float* partials
     return 0;
   }
   const dim3 grid(tokens, std::max(1, std::min((hidden + 255) / 256, 512 / tokens)));
-  if (weight_dtype == MK_F32)
-    norm_scale_add_kernel<float><<<grid, 256, 0, stream>>>(h, y, partials, count, (size_t)stride,
-                                                              weight, scale, eps, hidden);
-  else
-    norm_scale_add_kernel<bf16_t><<<grid, 256, 0, stream>>>(h, y, partials, count, (size_t)stride,
-                                                               weight, scale, eps, hidden);
+#define NSA_WIDE(TW)                                                                           \
+  do {                                                                                         \
+    if (x_bf16)                                                                                \
+      norm_scale_add_kernel<TW, bf16_t><<<grid, 256, 0, stream>>>(                             \
+          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden, (bf16_t*)x_out);  \
+    else                                                                                       \
+      norm_scale_add_kernel<TW, float><<<grid, 256, 0, stream>>>(                              \
+          h, y, partials, count, (size_t)stride, weight, scale, eps, hidden, (float*)x_out);   \
+  } while (0)
+  if (weight_dtype == MK_F32) NSA_WIDE(float);
+  else NSA_WIDE(bf16_t);
+#undef NSA_WIDE
   MK_LAUNCH_CHECK("norm_scale_add");
   return 0;
 }

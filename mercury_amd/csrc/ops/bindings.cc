@@ -384,7 +384,7 @@ void bind_ops(py::module_& m) {
     return blob(p);
   });
   m.def("post_norm_params", [](const std::string& kind_name, const py::bytes& sub, uintptr_t weight,
-                               int weight_dtype, uintptr_t scale, float eps) {
+                               int weight_dtype, uintptr_t scale, float eps, bool gives_x) {
     const OpKind& kind = OpRegistry::instance().get(kind_name);
     if (kind.flags & MK_OP_FOLDS_PENDING) {
       throw KernelError("the sublayer of a post norm cannot be an operation that adds up partial sums");
@@ -394,6 +394,7 @@ void bind_ops(py::module_& m) {
     p.weight = as_ptr<const void>(weight);
     p.weight_dtype = weight_dtype;
     p.scale = as_ptr<const float>(scale);
+    p.gives_x = gives_x ? 1 : 0;
     p.run = kind.run;
     p.tiles = kind.tiles;
     p.flags = kind.flags;
@@ -404,8 +405,9 @@ void bind_ops(py::module_& m) {
     std::memcpy(&out[0], &p, sizeof p);
     return py::bytes(out);
   }, py::arg("kind"), py::arg("sublayer"), py::arg("weight"), py::arg("weight_dtype"),
-     py::arg("scale") = 0, py::arg("eps") = 0.f,
-     "The parameter block of a 'post_norm' operation around one sublayer (kind, parameter bytes).");
+     py::arg("scale") = 0, py::arg("eps") = 0.f, py::arg("gives_x") = false,
+     "The parameter block of a 'post_norm' operation around one sublayer (kind, parameter bytes); "
+     "with gives_x the new stream goes out as x too, for an operation that reads the stream itself.");
   m.def("normed_sum_params", [](float mult, float eps, int weight_dtype,
                                  const std::vector<std::tuple<std::string, py::bytes, uintptr_t>>& subs) {
     if (subs.empty() || (int)subs.size() > kNormedSumMax) {

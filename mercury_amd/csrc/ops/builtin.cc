@@ -316,8 +316,14 @@ int run_post_norm(const void* params, mk_op_context* ctx) {
   ctx->out_logits_ready = 0;
   return guarded(ctx, [&] {
     Launch l(ctx);
+    void* x = p.gives_x ? l.alloc((size_t)tokens * ctx->hidden * l.elem()) : nullptr;
     norm_scale_add(l, h, y, parts, count, p.weight, p.weight_dtype, p.scale, p.eps, tokens,
-                   ctx->hidden);
+                   ctx->hidden, x);
+    if (p.gives_x) {
+      ctx->out_x = x;
+      ctx->out_x_rows = tokens;
+      ctx->out_x_live = 1;
+    }
   });
 }
 

@@ -77,6 +77,8 @@ struct PostNormParams {
   int weight_dtype = 0;
   const void* weight = nullptr;
   const float* scale = nullptr;     // float32 [hidden], or null
+  int gives_x = 0;                  // the new stream goes out as x too, in the compute dtype,
+                                    // for an operation behind this one that reads the stream itself
   mk_op_run_fn run = nullptr;
   mk_op_tiles_fn tiles = nullptr;
   int flags = 0;

@@ -499,11 +499,11 @@ void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float
 
 void norm_scale_add(Launch& l, float* h, const float* y, const float* partials, int count,
                     const void* weight, int weight_dtype, const float* scale, float eps,
-                    int tokens, int hidden) {
+                    int tokens, int hidden, void* x_out) {
   if (l.dry() || tokens == 0) return;
   check_core(need_core().mk_norm_scale_add(h, y, partials, count, (long long)tokens * hidden,
                                            weight, weight_dtype, scale, eps, tokens, hidden,
-                                           l.stream()), "norm_scale_add");
+                                           x_out, l.dtype(), l.stream()), "norm_scale_add");
 }
 
 void retention(Launch& l, const void* x, int m, int hidden, const RetentionArgs& a,

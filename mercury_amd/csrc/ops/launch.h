@@ -246,9 +246,10 @@ void* diff_heads(Launch& l, const void* a, int m, int heads, int dv, const float
                  int gate_stride, float lambda, float eps, float out_scale);
 
 // h += scale .* (rmsnorm(y + its partial sums) * weight) (see mk_norm_scale_add).
+// With `x_out` the new h also goes there, in the compute dtype.
 void norm_scale_add(Launch& l, float* h, const float* y, const float* partials, int count,
                     const void* weight, int weight_dtype, const float* scale, float eps,
-                    int tokens, int hidden);
+                    int tokens, int hidden, void* x_out = nullptr);
 
 // Retention: one projection [q | k | v | gate] in float32, the decayed recurrence per head from
 // the state earlier steps left (queries and keys turned, keys scaled), a norm per head, the

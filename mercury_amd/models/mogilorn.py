@@ -85,9 +85,12 @@ def build_mogilorn(cfg: MogilornConfig) -> DecoderModel:
                 out_gate=True)
             calls.append(LayerCall(i, i))
         ffn = UnaryMLP(cfg.width, entry.ff, "gelu_tanh", names=FF_NAMES) if entry.ff else None
+        # (the norm behind a sublayer hands the new stream on in the compute dtype: only the
+        # first layer copies it out by itself)
         layers.append(PrePostNormBlock(mixer, ffn, NoNorm(cfg.width), NoNorm(cfg.width) if ffn else None,
                                        post(), post() if ffn else None, BLOCK_NAMES,
-                                       layer_scale=False))
+                                       layer_scale=False, stream_given=i > 0,
+                                       next_reads_stream=i + 1 < len(cfg.layers)))
     return DecoderModel(
         vocab_size=cfg.vocab, hidden_size=cfg.width, layers=layers,
         final_norm=RMSNorm(cfg.width, cfg.norm_eps, one_plus=True), tied_head=True, calls=calls,

@@ -100,7 +100,14 @@ class PrePostNormBlock(Part):
 
     def __init__(self, mixer: Mixer, ffn: FeedForward | None, norm_mixer: Norm,
                  norm_ffn: Norm | None, post_mixer: Norm, post_ffn: Norm | None, names: dict,
-                 layer_scale: bool = True):
+                 layer_scale: bool = True, stream_given: bool = False,
+                 next_reads_stream: bool = False):
+        # Sublayers that read the stream itself (a `NoNorm` before them) need it in the compute
+        # dtype: the norm behind the sublayer before writes it out with the new stream, where
+        # there is one.  `stream_given`: the layer before this one does so for this layer's
+        # mixer (built with `next_reads_stream`); both concern the model's program only, a layer
+        # that runs alone makes its own copy.
+        self.stream_given, self.next_reads_stream = bool(stream_given), bool(next_reads_stream)
         self.mixer, self.ffn = mixer, ffn
         self.norm_mixer, self.norm_ffn = norm_mixer, norm_ffn
         self.post_mixer, self.post_ffn = post_mixer, post_ffn
@@ -129,7 +136,7 @@ class PrePostNormBlock(Part):
             return False
         return all(part.can_lower() for _, part in self._children())
 
-    def _wrapped(self, program, sub: "_Recorder", post: Norm, scale) -> None:
+    def _wrapped(self, program, sub: "_Recorder", post: Norm, scale, gives_x: bool = False) -> None:
         if len(sub.ops) != 1:
             raise ValueError("a sublayer between two norms lowers itself to one operation")
         if getattr(sub, "carried", 0):
@@ -138,21 +145,30 @@ class PrePostNormBlock(Part):
             raise ValueError("the norm behind a sublayer has no weight yet")
         program.append("post_norm", core.post_norm_params(
             sub.ops[0][0], sub.ops[0][1], post.weight.data_ptr(), ops.dtype_code(post.weight.dtype),
-            0 if scale is None else scale.data_ptr(), post.eps))
+            0 if scale is None else scale.data_ptr(), post.eps, gives_x=gives_x))
 
-    def lower(self, program, cache, state=None) -> None:
-        self.norm_mixer.lower(program)
+    def lower(self, program, cache, state=None, alone: bool = False) -> None:
+        from .norm import NoNorm
+
+        reads_stream = lambda norm: isinstance(norm, NoNorm)
+        if alone or not (self.stream_given and reads_stream(self.norm_mixer)):
+            self.norm_mixer.lower(program)
         sub = _Recorder()
         if state is None:
             self.mixer.lower(sub, cache)
         else:
             self.mixer.lower(sub, cache, state)
-        self._wrapped(program, sub, self.post_mixer, self.scale_mixer)
-        if self.ffn is not None:
+        hands_on = not alone and self.next_reads_stream
+        if self.ffn is None:
+            self._wrapped(program, sub, self.post_mixer, self.scale_mixer, gives_x=hands_on)
+            return
+        within = reads_stream(self.norm_ffn)
+        self._wrapped(program, sub, self.post_mixer, self.scale_mixer, gives_x=within)
+        if not within:
             self.norm_ffn.lower(program)
-            sub = _Recorder()
-            self.ffn.lower(sub)
-            self._wrapped(program, sub, self.post_ffn, self.scale_ffn)
+        sub = _Recorder()
+        self.ffn.lower(sub)
+        self._wrapped(program, sub, self.post_ffn, self.scale_ffn, gives_x=hands_on)
 
     def param_specs(self) -> dict:
         from .base import TensorSpec
@@ -192,8 +208,8 @@ class PrePostNormBlock(Part):
         key = (None if cache is None else cache.k.data_ptr(), None if state is None else state.data_ptr())
         alone = self._alone.get(key)
         if alone is None:
-            alone = self._alone[key] = OneOp(dtype, h.shape[1], 0,
-                                             lambda program: self.lower(program, cache, state))
+            alone = self._alone[key] = OneOp(
+                dtype, h.shape[1], 0, lambda program: self.lower(program, cache, state, alone=True))
         _logits, _x, left = alone.run(step, h, pending=pending)
         return left
 
