@@ -101,6 +101,10 @@ ATTENTION_SIZES = {
     "one-head-wide-values": (64, attention(1, 1, 8, 24, 0.35, softcap=3.0, rot=(100.0, 2))),
     "equal-widths-64": (128, attention(4, 2, 64, 64, 0.125, softcap=30.0, rot=(10000.0, 64), scaling=SCALING)),
     "equal-widths-128": (256, attention(2, 1, 128, 128, 0.09, softcap=20.0, rot=(10000.0, 128))),
+    "equal-widths-64-no-bound": (128, attention(4, 2, 64, 64, 0.125, rot=(10000.0, 32))),
+    "equal-widths-32": (64, attention(4, 4, 32, 32, 0.18, softcap=10.0, rot=(1000.0, 32), scaling=SCALING)),
+    "equal-widths-96": (96, attention(2, 1, 96, 96, 0.1, softcap=25.0, rot=(10000.0, 48))),
+    "equal-widths-80-no-bound": (80, attention(2, 2, 80, 80, 0.11)),
 }
 
 
