@@ -961,9 +961,10 @@ class MogilornConfig:
         mixing = self.mixing_layers()
         for i in mixing[1:]:
             first, m = self.layers[mixing[0]].mixer, self.layers[i].mixer
-            if (m.kv_heads, m.vdim) != (first.kv_heads, first.vdim):
+            # (the blend runs over a token's value columns side by side: as many are needed)
+            if m.kv_heads * m.vdim != first.kv_heads * first.vdim:
                 raise ConfigError(f"layers[{i}].mixer mixes its values with layer {mixing[0]}'s, "
-                                  "which has other kv_heads or vdim")
+                                  "which has another number of value columns (kv_heads * vdim)")
 
     def to_dict(self) -> dict:
         return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
